@@ -1,0 +1,109 @@
+/*
+ * kx_hip.h - C ABI of the MI355X (gfx950) kernels behind the kuiper matmul operator.
+ *
+ * This is the only place where host C++ meets HIP.  Plain pointers and sizes; no C++
+ * types, no torch types.  Every pointer is a DEVICE pointer unless said otherwise.
+ * `stream` is a hipStream_t passed as void* (nullptr = the default stream), exactly how the
+ * reference hands its stream to a kernel wrapper (kuiper/source/op/kernel/cuda/add_kernel.cu:28-48).
+ *
+ * Conventions shared by every entry point:
+ *   - returns 0 on success, a positive hipError_t if a HIP call failed, or a negative
+ *     KX_ERR_* code if the arguments were rejected before anything was launched;
+ *   - never synchronises, never allocates, never frees; work is enqueued on `stream`;
+ *   - 16-bit floats are passed as uint16_t bit patterns (bf16 activations / outputs,
+ *     fp16 scales).
+ *
+ * Packed AWQ layout (group size G along K, G a multiple of 32, K a multiple of G, N of 8):
+ *   qweight  int32 [K,   N/8]   nibble i (bits 4i..4i+3) of word (k, j) = code of column 8j+ORDER[i]
+ *   qzeros   int32 [K/G, N/8]   same nibble order
+ *   scales   fp16  [K/G, N]
+ *   ORDER = {0, 2, 4, 6, 1, 3, 5, 7}
+ * Dequantised weight: w[k,n] = (q[k,n] - z[k/G,n]) * s[k/G,n].
+ *
+ * The reference declares the operator these kernels serve but leaves it empty
+ * (kuiper/include/op/matmul.h:7-9, layer slot LayerMatmul kuiper/include/op/layer.h:14); the
+ * entry points below are what a kernel_interface entry in the style of
+ * kuiper/source/op/kernel/kernel_interface.h:10-11 binds to.
+ */
+#ifndef KX_HIP_H
+#define KX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KX_OK 0
+#define KX_ERR_NULL_POINTER (-1)   /* a required pointer is null */
+#define KX_ERR_BAD_SHAPE (-2)      /* M/K/N/group outside what the kernels accept */
+#define KX_ERR_WORKSPACE (-3)      /* workspace missing or smaller than kx_gemv_*_workspace_bytes */
+#define KX_ERR_ALIGNMENT (-4)      /* a pointer is not aligned as documented */
+
+#define KX_MAX_BATCH 16            /* largest M the GEMV entry points take */
+
+/* ABI version; bumped when a signature changes. */
+int kx_abi_version(void);
+
+/* Static, human-readable text for a return code of this library (KX_ERR_* or hipError_t). */
+const char* kx_error_string(int code);
+
+/* ------------------------------------------------------------------------------------------
+ * Workspace.  The fused GEMVs split K across workgroups; partial sums and per-tile arrival
+ * counters live in a caller-owned device buffer so that the GEMV itself never allocates.
+ *
+ *   bytes = kx_gemv_workspace_bytes(M, K, N)      (same figure serves both GEMV kinds)
+ *   kx_workspace_init(ws, bytes, stream)           once after allocation (zeroes the counters)
+ *
+ * A GEMV leaves the counters zeroed again, so one initialised workspace serves any number of
+ * consecutive launches on ONE stream.  Launches that may overlap (different streams) need
+ * separate workspaces.  The buffer must be 256-byte aligned.
+ * Reference counterpart: none (the reference has no split reduction); the allocator that
+ * would provide the buffer is base::CUDADeviceAllocator, kuiper/source/base/alloc_cu.cpp:8-16.
+ * ------------------------------------------------------------------------------------------ */
+size_t kx_gemv_workspace_bytes(int32_t M, int32_t K, int32_t N);
+int kx_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused INT4 AWQ dequantise + GEMV:   y[m,n] = sum_k x[m,k] * (q[k,n] - z[k/G,n]) * s[k/G,n]
+ *   x bf16 [M,K] row-major, y bf16 [M,N] row-major, fp32 accumulation, 1 <= M <= KX_MAX_BATCH.
+ *   Deterministic: the reduction order is fixed by (M,K,N,G), so repeated launches are bitwise
+ *   identical.  qweight/qzeros 4-byte aligned, scales 16-byte aligned, x 4-byte aligned.
+ * Replaces: the GPU branch of the quantised matmul kernel that the reference's MatmulLayer
+ * would fetch through kernel::get_matmul_kernel_awq(DeviceCUDA) (pattern:
+ * kuiper/source/op/kernel/kernel_interface.cpp:6-14, call site pattern kuiper/source/op/add.cpp:47).
+ * ------------------------------------------------------------------------------------------ */
+int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
+                     const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
+                     int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * BF16 GEMV fallback (non-quantised layers, lm_head):   y[m,n] = sum_k x[m,k] * W[n,k]
+ *   W bf16 [N,K] row-major (dim0 = output features, dim1 = input features, the reading of
+ *   LayerParam weights as [dim0, dim1]: kuiper/source/op/layer.cpp:256-276), K a multiple of 8,
+ *   W and x 16-byte aligned, 1 <= M <= KX_MAX_BATCH.  The workspace is not used by the current
+ *   kernels and may be null.
+ * Replaces: the GPU branch of kernel::get_matmul_kernel(DeviceCUDA) for an unquantised
+ * MatmulLayer (same dispatch pattern as above).
+ * ------------------------------------------------------------------------------------------ */
+int kx_gemv_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int32_t M, int32_t K,
+                 int32_t N, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Export kernels used to prove the integer side of the path bit-exactly.
+ *   kx_awq_unpack_u8     words int32 [rows, cols/8] -> codes uint8 [rows, cols] (values 0..15)
+ *   kx_awq_dequant_bf16  -> w bf16 [K,N], w = bf16_rne(float(q - z) * float(s)); the product is
+ *                           exact in fp32, so this has exactly one rounding.
+ * Reference counterpart: none; they serve the same checking role as the reference's GPU test
+ * helper test/utils.cu:19-38 (a kernel that exists for tests to read results back).
+ * ------------------------------------------------------------------------------------------ */
+int kx_awq_unpack_u8(const int32_t* words, uint8_t* codes, int64_t rows, int64_t cols,
+                     void* stream);
+int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
+                        uint16_t* w, int32_t K, int32_t N, int32_t group_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KX_HIP_H */

@@ -1,0 +1,112 @@
+"""ctypes binding of the C ABI in include/kx_hip.h.
+
+Device memory comes from torch tensors (plumbing only): the binding passes `tensor.data_ptr()`
+and torch's current HIP stream.  There is no fallback: if libkx_hip.so is missing, loading
+raises, and every entry point turns a non-zero return code into an exception.
+"""
+import ctypes
+import os
+
+from .build import KX_LIB
+
+_P = ctypes.c_void_p
+_I32 = ctypes.c_int32
+_I64 = ctypes.c_int64
+_SZ = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/kx_hip.h declaration by declaration
+SIGNATURES = {
+    "kx_abi_version": (ctypes.c_int, []),
+    "kx_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "kx_gemv_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "kx_workspace_init": (ctypes.c_int, [_P, _SZ, _P]),
+    "kx_gemv_awq_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
+    "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
+}
+
+
+class KxError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"kx call failed with code {code}: {text}")
+        self.code = code
+
+
+_lib = None
+
+
+def load():
+    """Load libkx_hip.so; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    # torch ships its own HIP runtime; it has to be in the process first so that this library
+    # binds to the same copy (two runtimes in one process do not share a device context).
+    import torch  # noqa: F401
+    if not os.path.exists(KX_LIB):
+        raise RuntimeError(
+            f"{KX_LIB} is missing: the HIP library has not been built "
+            "(python -m mykuiperllama_amd.build). There is no CPU fallback for this path.")
+    lib = ctypes.CDLL(KX_LIB)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _check(code):
+    if code != 0:
+        raise KxError(code, load().kx_error_string(code).decode())
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def workspace_bytes(M, K, N):
+    return int(load().kx_gemv_workspace_bytes(M, K, N))
+
+
+def make_workspace(M, K, N, device="cuda"):
+    """Allocate and initialise a workspace large enough for a GEMV of this shape."""
+    import torch
+    nbytes = max(workspace_bytes(M, K, N), 16384)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    _check(load().kx_workspace_init(ws.data_ptr(), nbytes, _stream()))
+    return ws
+
+
+def gemv_awq_bf16(x, qweight, scales, qzeros, y, group_size, workspace):
+    """x bf16 [M,K], qweight int32 [K,N/8], scales fp16 [K/G,N], qzeros int32 [K/G,N/8], y bf16 [M,N]."""
+    M, K = x.shape
+    N = y.shape[-1]
+    _check(load().kx_gemv_awq_bf16(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
+                                   M, K, N, group_size, _ptr(workspace),
+                                   0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_bf16(x, w, y, workspace=None):
+    """x bf16 [M,K], w bf16 [N,K], y bf16 [M,N]."""
+    M, K = x.shape
+    N = w.shape[0]
+    _check(load().kx_gemv_bf16(_ptr(x), _ptr(w), _ptr(y), M, K, N, _ptr(workspace),
+                               0 if workspace is None else workspace.numel(), _stream()))
+
+
+def awq_unpack_u8(words, codes):
+    rows, wcols = words.shape
+    _check(load().kx_awq_unpack_u8(_ptr(words), _ptr(codes), rows, wcols * 8, _stream()))
+
+
+def awq_dequant_bf16(qweight, scales, qzeros, w, group_size):
+    K, wcols = qweight.shape
+    _check(load().kx_awq_dequant_bf16(_ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(w), K,
+                                      wcols * 8, group_size, _stream()))

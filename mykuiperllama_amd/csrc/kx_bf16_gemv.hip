@@ -1,0 +1,105 @@
+// BF16 GEMV fallback for gfx950: y[m,n] = sum_k x[m,k] * W[n,k], W bf16 row-major [N, K].
+//
+// One wave per output row: the 64 lanes walk the row in 16-byte pieces (eight bf16 each), pairs
+// along K go through the packed bf16 dot instruction with an fp32 accumulator, and the lanes
+// meet in a butterfly at the end.  Rows are contiguous, so every load is a full 1 KiB per wave.
+#include "kx_common.h"
+
+namespace kx {
+namespace {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    bf16x2 va, vb;
+    __builtin_memcpy(&va, &a, 4);
+    __builtin_memcpy(&vb, &b, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(va, vb, c, false);
+}
+
+constexpr int kRowsPerBlock = 4;  // one wave each
+constexpr int kUnroll = 4;        // 16-byte loads in flight per lane
+
+template <int MB>
+__global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+    int M, int K, int N, int m0) {
+    const int lane = threadIdx.x % kWave;
+    const int n = blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
+    if (n >= N) return;
+    const int chunks = K >> 3;  // 16-byte pieces per row
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(w + static_cast<size_t>(n) * K);
+
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc[m] = 0.0f;
+
+    for (int c0 = lane; c0 < chunks; c0 += kWave * kUnroll) {
+        u32x4 wv[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const int c = c0 + u * kWave;
+            wv[u] = c < chunks ? __builtin_nontemporal_load(wrow + c) : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const int c = c0 + u * kWave;
+            if (c < chunks) {
+#pragma unroll
+                for (int m = 0; m < MB; m++) {
+                    if (m0 + m < M) {
+                        const uint4 xv = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + m) * K)[c];
+                        acc[m] = dot2_bf16(wv[u].x, xv.x, acc[m]);
+                        acc[m] = dot2_bf16(wv[u].y, xv.y, acc[m]);
+                        acc[m] = dot2_bf16(wv[u].z, xv.z, acc[m]);
+                        acc[m] = dot2_bf16(wv[u].w, xv.w, acc[m]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            acc[m] += __shfl_xor(acc[m], off, kWave);
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            if (m0 + m < M) y[static_cast<size_t>(m0 + m) * N + n] = f32_to_bf16(acc[m]);
+        }
+    }
+}
+
+}  // namespace
+}  // namespace kx
+
+extern "C" int kx_gemv_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int32_t M, int32_t K,
+                            int32_t N, void* workspace, size_t workspace_bytes, void* stream) {
+    (void)workspace;
+    (void)workspace_bytes;
+    if (!x || !w || !y) return KX_ERR_NULL_POINTER;
+    if (M < 1 || M > KX_MAX_BATCH || K < 8 || (K % 8) != 0 || N < 1) return KX_ERR_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(w) % 16 ||
+        reinterpret_cast<uintptr_t>(y) % 2) {
+        return KX_ERR_ALIGNMENT;
+    }
+    hipStream_t s = kx::as_stream(stream);
+    dim3 grid((N + kx::kRowsPerBlock - 1) / kx::kRowsPerBlock);
+    dim3 block(kx::kRowsPerBlock * kx::kWave);
+    for (int m0 = 0; m0 < M; m0 += 4) {
+        const int mb = M - m0 >= 4 ? 4 : (M - m0 >= 2 ? 2 : 1);
+        if (mb == 4) {
+            hipLaunchKernelGGL((kx::bf16_gemv_kernel<4>), grid, block, 0, s, x, w, y, M, K, N, m0);
+        } else if (mb == 2) {
+            hipLaunchKernelGGL((kx::bf16_gemv_kernel<2>), grid, block, 0, s, x, w, y, M, K, N, m0);
+            m0 -= 2;  // step of 4 below; a 2-row pass advances by 2
+        } else {
+            hipLaunchKernelGGL((kx::bf16_gemv_kernel<1>), grid, block, 0, s, x, w, y, M, K, N, m0);
+            m0 -= 3;
+        }
+    }
+    return kx::launch_status();
+}
