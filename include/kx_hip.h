@@ -69,7 +69,7 @@ int kx_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
  * Fused INT4 AWQ dequantise + GEMV:   y[m,n] = sum_k x[m,k] * (q[k,n] - z[k/G,n]) * s[k/G,n]
  *   x bf16 [M,K] row-major, y bf16 [M,N] row-major, fp32 accumulation, 1 <= M <= KX_MAX_BATCH.
  *   Deterministic: the reduction order is fixed by (M,K,N,G), so repeated launches are bitwise
- *   identical.  qweight/qzeros 4-byte aligned, scales 16-byte aligned, x 4-byte aligned.
+ *   identical.  qweight/qzeros 4-byte aligned, scales and x 16-byte aligned, y 8-byte aligned.
  * Replaces: the GPU branch of the quantised matmul kernel that the reference's MatmulLayer
  * would fetch through kernel::get_matmul_kernel_awq(DeviceCUDA) (pattern:
  * kuiper/source/op/kernel/kernel_interface.cpp:6-14, call site pattern kuiper/source/op/add.cpp:47).

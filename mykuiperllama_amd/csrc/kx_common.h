@@ -14,9 +14,11 @@ constexpr int kWave = 64;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-// Workspace layout: [kCounterBytes of uint32 arrival counters][fp32 partial sums].
-constexpr size_t kCounterBytes = 16384;
-constexpr int kMaxTiles = kCounterBytes / sizeof(uint32_t);
+// Workspace layout: [kCounterBytes of arrival counters, one per 64-byte line][fp32 partial sums].
+// Counters that share a line serialise at the memory side (~10 ns per atomic, measured), so
+// every (column tile, activation tile) pair gets a line of its own.
+constexpr size_t kCounterBytes = 65536;
+constexpr int kMaxTiles = kCounterBytes / 64;
 
 // nibble i of a packed word holds column 8j + kOrder[i]
 __host__ __device__ constexpr int order_of(int i) {

@@ -144,7 +144,7 @@ def test_linearity_in_x_at_full_size(capi, torch):
 
 
 def test_bad_arguments_are_rejected_before_launch(capi, torch):
-    p = synth.make_awq_problem("bad", 1, 256, 64)
+    p = synth.make_awq_problem("bad", 1, 1024, 64)
     x = H.to_dev_bf16(p["x"], torch)
     qw = H.to_dev_i32(p["qweight"], torch)
     sc = H.to_dev_f16(p["scales"], torch)
@@ -153,10 +153,29 @@ def test_bad_arguments_are_rejected_before_launch(capi, torch):
     L = capi.load()
     s = torch.cuda.current_stream().cuda_stream
     args = (x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr())
-    assert L.kx_gemv_awq_bf16(*args, 1, 256, 64, 128, None, 0, s) == -3      # needs a workspace
-    assert L.kx_gemv_awq_bf16(*args, 0, 256, 64, 128, None, 0, s) == -2      # M = 0
-    assert L.kx_gemv_awq_bf16(*args, 17, 256, 64, 128, None, 0, s) == -2     # M too large
-    assert L.kx_gemv_awq_bf16(*args, 1, 250, 64, 128, None, 0, s) == -2      # K not a group multiple
-    assert L.kx_gemv_awq_bf16(*args, 1, 256, 60, 128, None, 0, s) == -2      # N not a multiple of 8
-    assert L.kx_gemv_awq_bf16(None, *args[1:], 1, 256, 64, 128, None, 0, s) == -1
+    small = torch.empty(65536 + 64, dtype=torch.uint8, device="cuda")
+    assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 128, None, 0, s) == -3     # K is split: needs a workspace
+    assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 128, small.data_ptr(), small.numel(), s) == -3  # too small
+    assert L.kx_gemv_awq_bf16(*args, 0, 1024, 64, 128, None, 0, s) == -2     # M = 0
+    assert L.kx_gemv_awq_bf16(*args, 17, 1024, 64, 128, None, 0, s) == -2    # M too large
+    assert L.kx_gemv_awq_bf16(*args, 1, 1000, 64, 128, None, 0, s) == -2     # K not a group multiple
+    assert L.kx_gemv_awq_bf16(*args, 1, 1024, 60, 128, None, 0, s) == -2     # N not a multiple of 8
+    assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 48, None, 0, s) == -2      # group not a multiple of 32
+    assert L.kx_gemv_awq_bf16(None, *args[1:], 1, 1024, 64, 128, None, 0, s) == -1
+    assert L.kx_gemv_awq_bf16(args[0] + 2, *args[1:], 1, 1024, 64, 128, None, 0, s) == -4  # x misaligned
+    assert capi.workspace_bytes(1, 1024, 64) > 65536
+    assert capi.workspace_bytes(0, 1024, 64) == 0
     torch.cuda.synchronize()
+
+
+def test_unsplit_k_needs_no_workspace(capi, torch, oracle):
+    """K that fits one workgroup is reduced without the exchange: a null workspace is accepted."""
+    p = synth.make_awq_problem("unsplit", 2, 256, 512)
+    x = H.to_dev_bf16(p["x"], torch)
+    qw = H.to_dev_i32(p["qweight"], torch)
+    sc = H.to_dev_f16(p["scales"], torch)
+    qz = H.to_dev_i32(p["qzeros"], torch)
+    y = torch.full((2, 512), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_bf16(x, qw, sc, qz, y, p["group"], None)
+    torch.cuda.synchronize()
+    check_against_oracle(oracle, p, H.bf16_bits(y, torch))
