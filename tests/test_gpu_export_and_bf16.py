@@ -101,3 +101,30 @@ def test_bf16_gemv_one_hot_returns_the_weight_column_exactly(capi, torch):
         capi.gemv_bf16(H.to_dev_bf16(xb, torch), w, y)
         torch.cuda.synchronize()
         assert np.array_equal(H.bf16_bits(y, torch)[0], p["w"][:, k])
+
+
+def test_gpu_reproduces_golden_fixture(capi, torch):
+    """The committed fixture (numpy restatement of the layout + torch's bf16 cast) end to end."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "awq_small.npz"))
+    group = int(g["group"])
+    K, N = g["codes"].shape
+    qw, qz = H.to_dev_i32(g["qweight"], torch), H.to_dev_i32(g["qzeros"], torch)
+    sc = H.to_dev_f16(g["scales"], torch)
+    codes = torch.zeros((K, N), dtype=torch.uint8, device="cuda")
+    capi.awq_unpack_u8(qw, codes)
+    zc = torch.zeros(tuple(g["zero_codes"].shape), dtype=torch.uint8, device="cuda")
+    capi.awq_unpack_u8(qz, zc)
+    w = torch.zeros((K, N), dtype=torch.bfloat16, device="cuda")
+    capi.awq_dequant_bf16(qw, sc, qz, w, group)
+    x = H.to_dev_bf16(g["x"], torch)
+    y = torch.zeros((x.shape[0], N), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_bf16(x, qw, sc, qz, y, group, capi.make_workspace(x.shape[0], K, N))
+    torch.cuda.synchronize()
+    assert np.array_equal(codes.cpu().numpy(), g["codes"])
+    assert np.array_equal(zc.cpu().numpy(), g["zero_codes"])
+    assert np.array_equal(H.bf16_bits(w, torch), g["w_bf16"])
+    got = H.bf16_to_f64(H.bf16_bits(y, torch))
+    ref = H.bf16_to_f64(synth.f32_to_bf16_bits(g["y_f64"].astype(np.float32)))
+    assert H.rel_l2(got, ref) <= 1e-3
+    assert np.abs(got - ref).max() <= 2 * H.bf16_ulp_of(np.abs(g["y_f64"]).max())
