@@ -2,7 +2,7 @@
 
   libkx_hip.so   HIP kernels + C ABI            (csrc/*.hip)
   libkuiper.so   C++ host API over that C ABI    (kuiper/source/**/*.cpp)
-  test_kuiper    C++ test runner for the host API (kuiper/test/*.cpp)
+  test_kuiper    C++ test runner for the host API (tests/cpp/*, links oracle/kx_oracle.c)
 
 Everything lands under mykuiperllama_amd/lib/, in-tree, so that a snapshot of the repository
 carries the binaries to a machine that only runs them.
@@ -17,6 +17,7 @@ LIB_DIR = os.path.join(PKG, "lib")
 CSRC = os.path.join(PKG, "csrc")
 KUIPER = os.path.join(PKG, "kuiper")
 INCLUDE = os.path.join(ROOT, "include")
+TESTS_CPP = os.path.join(ROOT, "tests", "cpp")
 
 KX_LIB = os.path.join(LIB_DIR, "libkx_hip.so")
 KUIPER_LIB = os.path.join(LIB_DIR, "libkuiper.so")
@@ -45,15 +46,26 @@ def build_kx():
 
 def build_kuiper():
     os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = sorted(glob.glob(os.path.join(KUIPER, "source", "**", "*.cpp"), recursive=True))
+    srcs = sorted(glob.glob(os.path.join(KUIPER, "source", "**", "*.cpp"), recursive=True) +
+                  glob.glob(os.path.join(KUIPER, "source", "**", "*.hip"), recursive=True))
     if not srcs:
         return None
     inc = ["-I", INCLUDE, "-I", os.path.join(KUIPER, "include"), "-I", os.path.join(KUIPER, "source", "op")]
     _run([HIPCC] + DEVICE_FLAGS + COMMON + ["-shared"] + inc + srcs +
          ["-L", LIB_DIR, "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", KUIPER_LIB])
-    tests = sorted(glob.glob(os.path.join(KUIPER, "test", "*.cpp")))
+    # C++ tests of the host API live under tests/cpp and link the CPU oracle as their checker
+    tests = sorted(glob.glob(os.path.join(TESTS_CPP, "*.cpp")) + glob.glob(os.path.join(TESTS_CPP, "*.hip")))
     if tests:
-        _run([HIPCC] + DEVICE_FLAGS + COMMON + inc + ["-I", os.path.join(KUIPER, "test")] + tests +
+        oracle_obj = os.path.join(LIB_DIR, "kx_oracle_for_tests.o")
+        _run(["gcc", "-O2", "-fPIC", "-std=c11", "-c", os.path.join(ROOT, "oracle", "kx_oracle.c"), "-o", oracle_obj])
+        objs = [oracle_obj]
+        obj_dir = os.path.join(LIB_DIR, "obj")
+        os.makedirs(obj_dir, exist_ok=True)
+        for src in tests:  # one object per source: hipcc would read a mixed .hip/.o line as all-HIP
+            obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+            _run([HIPCC] + DEVICE_FLAGS + COMMON + inc + ["-I", TESTS_CPP, "-c", src, "-o", obj])
+            objs.append(obj)
+        _run([HIPCC, "--offload-arch=gfx950"] + objs +
              ["-L", LIB_DIR, "-lkuiper", "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", KUIPER_TEST])
     return KUIPER_LIB
 

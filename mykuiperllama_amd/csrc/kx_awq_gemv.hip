@@ -17,9 +17,6 @@ inline int rows_per_block(int waves, int rt) {
     return waves * kSlotsPerWave * rt;
 }
 
-// The smallest slice of K a workgroup may take; bounds the number of partial sums.
-constexpr int kMinRowsPerBlock = 4 * kSlotsPerWave * 8;
-
 inline AwqPlan make_plan(int M, int K, int N) {
     AwqPlan p;
     p.mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
@@ -61,9 +58,8 @@ __global__ void fill_zero_u32(uint32_t* p, size_t n) {
 
 extern "C" size_t kx_gemv_workspace_bytes(int32_t M, int32_t K, int32_t N) {
     if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8) return 0;
-    // Upper bound over every plan: the smallest workgroup slice of K gives the most partials.
-    size_t ktiles = (static_cast<size_t>(K) + kx::kMinRowsPerBlock - 1) / kx::kMinRowsPerBlock;
-    return kx::kCounterBytes + ktiles * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+    const kx::AwqPlan p = kx::make_plan(M, K, N);
+    return kx::kCounterBytes + static_cast<size_t>(p.ktiles) * M * static_cast<size_t>(N) * sizeof(float);
 }
 
 extern "C" int kx_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {

@@ -1,0 +1,110 @@
+// GPU side of the matmul operator: tensors in, C ABI out.
+#include "matmul_kernel.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <memory>
+
+#include "kx_hip.h"
+
+namespace kernel {
+namespace {
+
+struct Workspace {
+    std::shared_ptr<base::Buffer> buffer;
+};
+
+// One workspace per stream: launches on one stream run in order and may share it, launches on
+// different streams may overlap and must not.  Single host thread assumed, like the rest of the
+// host API.
+std::map<void*, Workspace>& workspaces() {
+    static std::map<void*, Workspace> table;
+    return table;
+}
+
+void* workspace_for(void* stream, size_t bytes) {
+    if (bytes == 0) {
+        return nullptr;
+    }
+    Workspace& ws = workspaces()[stream];
+    if (ws.buffer == nullptr || ws.buffer->byte_size() < bytes) {
+        if (ws.buffer != nullptr) {
+            // the old buffer may still be in use by launches already enqueued on this stream
+            (void)hipStreamSynchronize(static_cast<hipStream_t>(stream));
+        }
+        ws.buffer = std::make_shared<base::Buffer>(bytes, base::CUDADeviceAllocatorFactory::get_instance());
+        CHECK_NE(ws.buffer->ptr(), nullptr);
+        const int rc = kx_workspace_init(ws.buffer->ptr(), bytes, stream);
+        CHECK_EQ(rc, KX_OK) << "workspace init failed: " << kx_error_string(rc);
+    }
+    return ws.buffer->ptr();
+}
+
+int32_t rows_of(const tensor::Tensor& t, int32_t inner) {
+    if (t.dims_size() == 1) {
+        CHECK_EQ(t.get_dim(0), inner);
+        return 1;
+    }
+    CHECK_EQ(t.dims_size(), 2);
+    CHECK_EQ(t.get_dim(1), inner);
+    return t.get_dim(0);
+}
+
+}  // namespace
+
+void matmul_release_workspaces() {
+    workspaces().clear();
+}
+
+void matmul_kernel_cu(const tensor::Tensor& input, const tensor::Tensor& weight,
+                      const tensor::Tensor& output, void* stream) {
+    CHECK(input.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(weight.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(output.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK_EQ(input.is_empty(), false);
+    CHECK_EQ(weight.is_empty(), false);
+    CHECK_EQ(output.is_empty(), false);
+    CHECK_EQ(weight.dims_size(), 2);
+    const int32_t N = weight.get_dim(0);
+    const int32_t K = weight.get_dim(1);
+    const int32_t M = rows_of(input, K);
+    CHECK_EQ(rows_of(output, N), M);
+
+    const int rc = kx_gemv_bf16(input.ptr<uint16_t>(), weight.ptr<uint16_t>(),
+                                const_cast<uint16_t*>(output.ptr<uint16_t>()), M, K, N, nullptr, 0, stream);
+    CHECK(rc == KX_OK) << "BF16 matmul kernel launch failed: " << kx_error_string(rc);
+}
+
+void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qweight,
+                          const tensor::Tensor& scales, const tensor::Tensor& qzeros,
+                          const tensor::Tensor& output, int32_t group_size, void* stream) {
+    CHECK(input.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(qweight.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(scales.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(qzeros.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK(output.device_type() == base::DeviceType::DeviceCUDA);
+    CHECK_EQ(input.is_empty(), false);
+    CHECK_EQ(qweight.is_empty(), false);
+    CHECK_EQ(scales.is_empty(), false);
+    CHECK_EQ(qzeros.is_empty(), false);
+    CHECK_EQ(output.is_empty(), false);
+    CHECK_EQ(qweight.dims_size(), 2);
+    CHECK_GT(group_size, 0);
+    const int32_t K = qweight.get_dim(0);
+    const int32_t N = qweight.get_dim(1) * 8;
+    CHECK_EQ(K % group_size, 0);
+    CHECK_EQ(scales.size(), static_cast<size_t>(K / group_size) * N);
+    CHECK_EQ(qzeros.size(), static_cast<size_t>(K / group_size) * (N / 8));
+    const int32_t M = rows_of(input, K);
+    CHECK_EQ(rows_of(output, N), M);
+
+    const size_t ws_bytes = kx_gemv_workspace_bytes(M, K, N);
+    void* ws = workspace_for(stream, ws_bytes);
+    const int rc = kx_gemv_awq_bf16(input.ptr<uint16_t>(), qweight.ptr<int32_t>(), scales.ptr<uint16_t>(),
+                                    qzeros.ptr<int32_t>(), const_cast<uint16_t*>(output.ptr<uint16_t>()), M, K,
+                                    N, group_size, ws, ws_bytes, stream);
+    CHECK(rc == KX_OK) << "AWQ matmul kernel launch failed: " << kx_error_string(rc);
+}
+
+}  // namespace kernel

@@ -1,0 +1,24 @@
+#ifndef KUIPER_KERNEL_HIP_MATMUL_KERNEL_H
+#define KUIPER_KERNEL_HIP_MATMUL_KERNEL_H
+
+#include "tensor/tensor.h"
+
+namespace kernel {
+
+// GPU kernels of the matmul operator: thin wrappers that check the tensors the way the
+// reference's GPU wrapper does (kuiper/source/op/kernel/cuda/add_kernel.cu:14-52: device, non-empty,
+// sizes; then launch; then a fatal check of the launch status; no synchronisation) and call the
+// C ABI of the HIP library (include/kx_hip.h).  The split-K workspace is kept per stream and
+// grows on demand; it is the only allocation these wrappers ever make.
+void matmul_kernel_cu(const tensor::Tensor& input, const tensor::Tensor& weight,
+                      const tensor::Tensor& output, void* stream);
+void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qweight,
+                          const tensor::Tensor& scales, const tensor::Tensor& qzeros,
+                          const tensor::Tensor& output, int32_t group_size, void* stream);
+
+// Releases every cached workspace (for orderly shutdown in tests).
+void matmul_release_workspaces();
+
+}  // namespace kernel
+
+#endif  // KUIPER_KERNEL_HIP_MATMUL_KERNEL_H

@@ -1,0 +1,266 @@
+// MatmulLayer and the matmul kernel-selection entries, against the CPU oracle
+// (oracle/kx_oracle.c, linked into this test binary as the checker).  Tolerances are the path's:
+// relative L2 <= 1e-3 against the oracle's value rounded to bf16, max-abs <= 2 bf16 ulp of the
+// output scale; one-hot activations must reproduce dequantised rows bit for bit.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "../../mykuiperllama_amd/kuiper/source/op/kernel/kernel_interface.h"
+#include "../../oracle/kx_oracle.h"
+#include "mini_test.h"
+#include "op/matmul.h"
+
+namespace {
+
+struct Rng {  // SplitMix64
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed) {}
+    uint64_t next() {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double uniform() { return double(next() >> 11) * (1.0 / 9007199254740992.0); }
+    double normal() { return std::sqrt(-2.0 * std::log(1.0 - uniform())) * std::cos(6.283185307179586 * uniform()); }
+};
+
+struct AwqProblem {
+    int M, K, N, G;
+    std::vector<uint16_t> x, scales;
+    std::vector<int32_t> qweight, qzeros;
+};
+
+AwqProblem make_problem(int M, int K, int N, int G, uint64_t seed) {
+    AwqProblem p{M, K, N, G, {}, {}, {}, {}};
+    Rng rng(seed);
+    p.x.resize(size_t(M) * K);
+    for (auto& v : p.x) v = kxo_f32_to_bf16(float(rng.normal()));
+    p.qweight.resize(size_t(K) * N / 8);
+    for (auto& v : p.qweight) v = int32_t(rng.next());
+    p.qzeros.resize(size_t(K / G) * N / 8);
+    for (auto& v : p.qzeros) v = int32_t(rng.next());
+    p.scales.resize(size_t(K / G) * N);
+    for (auto& v : p.scales) v = kxo_f32_to_f16(float(0.001 + 0.019 * rng.uniform()));
+    return p;
+}
+
+double bf16_ulp(double v) { return std::pow(2.0, std::floor(std::log2(v)) - 7); }
+
+// got: bf16 [M, N]; ref: fp64 [M, N]
+void expect_close(const std::vector<uint16_t>& got, const std::vector<double>& ref) {
+    double num = 0, den = 0, maxabs = 0, maxerr = 0;
+    for (size_t i = 0; i < ref.size(); i++) {
+        const double r = kxo_bf16_to_f32(kxo_f32_to_bf16(float(ref[i])));
+        const double g = kxo_bf16_to_f32(got[i]);
+        ASSERT_TRUE(std::isfinite(g));
+        num += (g - r) * (g - r);
+        den += r * r;
+        maxabs = std::fmax(maxabs, std::fabs(ref[i]));
+        maxerr = std::fmax(maxerr, std::fabs(g - r));
+    }
+    ASSERT_LE(std::sqrt(num / den), 1e-3);
+    ASSERT_LE(maxerr, 2 * bf16_ulp(maxabs));
+}
+
+template <typename T>
+tensor::Tensor host_tensor(base::DataType type, std::vector<int32_t> dims, std::vector<T>& data) {
+    tensor::Tensor t(type, std::move(dims), false, nullptr, data.data());
+    t.set_device_type(base::DeviceType::DeviceCPU);
+    return t;
+}
+
+// Builds an AWQ layer on `device` from host data (moved to the GPU when asked) and runs it.
+std::vector<uint16_t> run_awq_layer(AwqProblem& p, base::DeviceType device, bool one_d_io = false) {
+    const bool gpu = device == base::DeviceType::DeviceCUDA;
+    op::MatmulLayer layer(device, p.N, p.K, true, p.G);
+    tensor::Tensor qw = host_tensor(base::DataType::DataTypeInt32, {p.K, p.N / 8}, p.qweight);
+    tensor::Tensor qz = host_tensor(base::DataType::DataTypeInt32, {p.K / p.G, p.N / 8}, p.qzeros);
+    tensor::Tensor sc = host_tensor(base::DataType::DataTypeFp16, {p.K / p.G, p.N}, p.scales);
+    tensor::Tensor x = one_d_io ? host_tensor(base::DataType::DataTypeBf16, {p.K}, p.x)
+                                : host_tensor(base::DataType::DataTypeBf16, {p.M, p.K}, p.x);
+    std::vector<uint16_t> out(size_t(p.M) * p.N, 0x7FC0);
+    tensor::Tensor y = one_d_io ? host_tensor(base::DataType::DataTypeBf16, {p.N}, out)
+                                : host_tensor(base::DataType::DataTypeBf16, {p.M, p.N}, out);
+    if (gpu) {
+        qw.to_cuda();
+        qz.to_cuda();
+        sc.to_cuda();
+        x.to_cuda();
+        y.to_cuda();
+        auto config = std::make_shared<kernel::CudaConfig>();
+        config->create();
+        layer.set_cuda_config(config);
+    }
+    ASSERT_TRUE(bool(layer.set_weight(0, qw)));
+    ASSERT_TRUE(bool(layer.set_weight(1, qz)));
+    layer.set_awq_scales(sc);
+    base::Status st = layer.forward(x, y);
+    ASSERT_TRUE(bool(st));
+    if (gpu) {
+        ASSERT_EQ(hipStreamSynchronize(layer.cuda_config()->stream()), hipSuccess);
+        y.to_cpu();
+        std::memcpy(out.data(), y.ptr<uint16_t>(), out.size() * 2);
+    }
+    return out;
+}
+
+std::vector<double> oracle_awq(const AwqProblem& p) {
+    std::vector<double> ref(size_t(p.M) * p.N);
+    ASSERT_EQ(kxo_gemv_awq_f64(p.x.data(), p.qweight.data(), p.scales.data(), p.qzeros.data(), p.M, p.K, p.N, p.G,
+                               ref.data()), 0);
+    return ref;
+}
+
+void awq_layer_matches_oracle(base::DeviceType device) {
+    const int shapes[][4] = {{1, 1024, 2048, 128}, {1, 4096, 1024, 128}, {4, 512, 264, 64}, {16, 256, 64, 128}};
+    for (const auto& s : shapes) {
+        AwqProblem p = make_problem(s[0], s[1], s[2], s[3], 1000 + s[0] + s[1]);
+        expect_close(run_awq_layer(p, device), oracle_awq(p));
+    }
+    AwqProblem p1 = make_problem(1, 512, 128, 128, 77);  // [K] in, [N] out
+    expect_close(run_awq_layer(p1, device, true), oracle_awq(p1));
+}
+
+void awq_one_hot_is_bit_exact(base::DeviceType device) {
+    AwqProblem p = make_problem(1, 512, 256, 128, 5);
+    std::vector<uint16_t> w(size_t(p.K) * p.N);
+    ASSERT_EQ(kxo_awq_dequant_bf16(p.qweight.data(), p.scales.data(), p.qzeros.data(), p.K, p.N, p.G, w.data()), 0);
+    for (int k : {0, 127, 128, 300, 511}) {
+        std::fill(p.x.begin(), p.x.end(), uint16_t(0));
+        p.x[k] = 0x3F80;
+        std::vector<uint16_t> y = run_awq_layer(p, device);
+        for (int n = 0; n < p.N; n++) ASSERT_EQ(y[n], w[size_t(k) * p.N + n]);
+    }
+}
+
+void bf16_layer_matches_oracle(base::DeviceType device) {
+    const bool gpu = device == base::DeviceType::DeviceCUDA;
+    const int M = 3, K = 1024, N = 515;
+    Rng rng(99);
+    std::vector<uint16_t> x(size_t(M) * K), w(size_t(N) * K), out(size_t(M) * N, 0x7FC0);
+    for (auto& v : x) v = kxo_f32_to_bf16(float(rng.normal()));
+    for (auto& v : w) v = kxo_f32_to_bf16(float(0.02 * rng.normal()));
+    std::vector<double> ref(size_t(M) * N);
+    ASSERT_EQ(kxo_gemv_bf16_f64(x.data(), w.data(), M, K, N, ref.data()), 0);
+    op::MatmulLayer layer(device, N, K);
+    ASSERT_EQ(layer.weights_size(), 1u);
+    tensor::Tensor xt = host_tensor(base::DataType::DataTypeBf16, {M, K}, x);
+    tensor::Tensor yt = host_tensor(base::DataType::DataTypeBf16, {M, N}, out);
+    if (gpu) {
+        // raw-pointer attach of device memory, the way a model loader hands weights over
+        auto alloc = base::CUDADeviceAllocatorFactory::get_instance();
+        static std::shared_ptr<base::Buffer> keep;
+        keep = std::make_shared<base::Buffer>(w.size() * 2, alloc);
+        alloc->memcpy(keep->ptr(), w.data(), w.size() * 2, base::MemcpyKind::MemcpyCPU2CUDA);
+        ASSERT_TRUE(bool(layer.set_weight(0, {N, K}, keep->ptr(), base::DeviceType::DeviceCUDA)));
+        xt.to_cuda();
+        yt.to_cuda();
+        auto config = std::make_shared<kernel::CudaConfig>();
+        config->create();
+        layer.set_cuda_config(config);
+    } else {
+        ASSERT_TRUE(bool(layer.set_weight(0, {N, K}, w.data(), base::DeviceType::DeviceCPU)));
+    }
+    ASSERT_TRUE(bool(layer.forward(xt, yt)));
+    if (gpu) {
+        ASSERT_EQ(hipDeviceSynchronize(), hipSuccess);
+        yt.to_cpu();
+        std::memcpy(out.data(), yt.ptr<uint16_t>(), out.size() * 2);
+    }
+    expect_close(out, ref);
+}
+
+}  // namespace
+
+TEST_CPU(test_matmul, awq_layer_cpu_matches_oracle) { awq_layer_matches_oracle(base::DeviceType::DeviceCPU); }
+TEST_GPU(test_matmul, awq_layer_cuda_matches_oracle) { awq_layer_matches_oracle(base::DeviceType::DeviceCUDA); }
+TEST_CPU(test_matmul, awq_layer_cpu_one_hot_bit_exact) { awq_one_hot_is_bit_exact(base::DeviceType::DeviceCPU); }
+TEST_GPU(test_matmul, awq_layer_cuda_one_hot_bit_exact) { awq_one_hot_is_bit_exact(base::DeviceType::DeviceCUDA); }
+TEST_CPU(test_matmul, bf16_layer_cpu_matches_oracle) { bf16_layer_matches_oracle(base::DeviceType::DeviceCPU); }
+TEST_GPU(test_matmul, bf16_layer_cuda_matches_oracle) { bf16_layer_matches_oracle(base::DeviceType::DeviceCUDA); }
+
+TEST_GPU(test_matmul, awq_full_size_projection_and_repeat_calls) {
+    AwqProblem p = make_problem(1, 4096, 4096, 128, 4242);
+    std::vector<uint16_t> first = run_awq_layer(p, base::DeviceType::DeviceCUDA);
+    expect_close(first, oracle_awq(p));
+    // the per-stream workspace is reused; results stay bitwise identical
+    for (int i = 0; i < 3; i++) ASSERT_EQ(run_awq_layer(p, base::DeviceType::DeviceCUDA), first);
+}
+
+TEST_CPU(test_matmul, layer_construction_and_checks) {
+    auto allocator = base::CPUDeviceAllocatorFactory::get_instance();
+    op::MatmulLayer quant(base::DeviceType::DeviceCPU, 64, 256, true);
+    ASSERT_TRUE(quant.layer_type() == op::LayerType::LayerMatmul);
+    ASSERT_TRUE(quant.data_type() == base::DataType::DataTypeBf16);
+    ASSERT_EQ(quant.weights_size(), 2u);
+    ASSERT_EQ(quant.group_size(), 128);
+    ASSERT_EQ(quant.dim0(), 64);
+    ASSERT_EQ(quant.dim1(), 256);
+    ASSERT_TRUE(quant.is_quant_layer());
+    tensor::Tensor x(base::DataType::DataTypeBf16, 1, 256, true, allocator);
+    tensor::Tensor y(base::DataType::DataTypeBf16, 1, 64, true, allocator);
+    // nothing attached yet: check() reports, forward() returns that status without aborting
+    base::Status st = quant.forward(x, y);
+    ASSERT_FALSE(bool(st));
+    ASSERT_EQ(int(st), int(base::StatusCode::InvalidArgument));
+    // element types are enforced per slot
+    tensor::Tensor f32(base::DataType::DataTypeFp32, 1, 256, true, allocator);
+    ASSERT_FATAL(quant.set_input(0, f32));
+    ASSERT_FATAL(quant.set_output(0, f32));
+    ASSERT_FATAL(quant.set_weight(0, f32));
+    ASSERT_FATAL(quant.set_awq_scales(f32));
+    ASSERT_FATAL(quant.set_weight(2, f32));
+    // wrong shapes are reported through the Status
+    tensor::Tensor qw(base::DataType::DataTypeInt32, 256, 8, true, allocator);
+    tensor::Tensor qz(base::DataType::DataTypeInt32, 2, 8, true, allocator);
+    tensor::Tensor sc(base::DataType::DataTypeFp16, 2, 64, true, allocator);
+    tensor::Tensor sc_bad(base::DataType::DataTypeFp16, 2, 63, true, allocator);
+    quant.set_weight(0, qw);
+    quant.set_weight(1, qz);
+    quant.set_awq_scales(sc_bad);
+    ASSERT_FALSE(bool(quant.forward(x, y)));
+    quant.set_awq_scales(sc);
+    std::memset(qw.ptr<void>(), 0, qw.byte_size());
+    std::memset(qz.ptr<void>(), 0, qz.byte_size());
+    std::memset(sc.ptr<void>(), 0, sc.byte_size());
+    std::memset(x.ptr<void>(), 0, x.byte_size());
+    ASSERT_TRUE(bool(quant.forward(x, y)));
+    tensor::Tensor x_bad(base::DataType::DataTypeBf16, 1, 255, true, allocator);
+    ASSERT_FALSE(bool(quant.forward(x_bad, y)));
+    tensor::Tensor x17(base::DataType::DataTypeBf16, 17, 256, true, allocator);
+    tensor::Tensor y17(base::DataType::DataTypeBf16, 17, 64, true, allocator);
+    ASSERT_FALSE(bool(quant.forward(x17, y17)));  // M beyond the decode-sized batch
+    tensor::Tensor y_bad(base::DataType::DataTypeBf16, 2, 64, true, allocator);
+    ASSERT_FALSE(bool(quant.forward(x, y_bad)));
+    // unquantised layer refuses scales
+    op::MatmulLayer plain(base::DeviceType::DeviceCPU, 64, 256);
+    ASSERT_EQ(plain.group_size(), 0);
+    ASSERT_FATAL(plain.set_awq_scales(sc));
+    // kernel selection
+    ASSERT_FATAL(kernel::get_matmul_kernel(base::DeviceType::DeviceUnknown));
+    ASSERT_FATAL(kernel::get_matmul_kernel_awq(base::DeviceType::DeviceUnknown));
+    // the GPU wrappers refuse host tensors before touching the device
+    ASSERT_FATAL(kernel::get_matmul_kernel_awq(base::DeviceType::DeviceCUDA)(x, qw, sc, qz, y, 128, nullptr));
+    ASSERT_FATAL(kernel::get_matmul_kernel(base::DeviceType::DeviceCUDA)(x, x, y, nullptr));
+}
+
+TEST_GPU(test_matmul, kernel_interface_direct_call_on_default_stream) {
+    // the function pointer is public interface: call it without a layer, stream = nullptr
+    AwqProblem p = make_problem(2, 1024, 512, 128, 31337);
+    tensor::Tensor qw = host_tensor(base::DataType::DataTypeInt32, {p.K, p.N / 8}, p.qweight);
+    tensor::Tensor qz = host_tensor(base::DataType::DataTypeInt32, {p.K / p.G, p.N / 8}, p.qzeros);
+    tensor::Tensor sc = host_tensor(base::DataType::DataTypeFp16, {p.K / p.G, p.N}, p.scales);
+    tensor::Tensor x = host_tensor(base::DataType::DataTypeBf16, {p.M, p.K}, p.x);
+    std::vector<uint16_t> out(size_t(p.M) * p.N, 0);
+    tensor::Tensor y = host_tensor(base::DataType::DataTypeBf16, {p.M, p.N}, out);
+    for (tensor::Tensor* t : {&qw, &qz, &sc, &x, &y}) t->to_cuda();
+    kernel::get_matmul_kernel_awq(base::DeviceType::DeviceCUDA)(x, qw, sc, qz, y, p.G, nullptr);
+    ASSERT_EQ(hipDeviceSynchronize(), hipSuccess);
+    y.to_cpu();
+    std::memcpy(out.data(), y.ptr<uint16_t>(), out.size() * 2);
+    expect_close(out, oracle_awq(p));
+}

@@ -1,0 +1,259 @@
+// Tensor semantics.  Restates the assertions of the reference's test/test_tensor/test_tensor.cpp
+// (tensor_base :6-19, clone_cuda :21-60, clone_cpu :62-80, to_cuda :82-100, init1..init6 :102-207,
+// dims_stride :226-247, assign :249-276) on this build's classes, plus host-side variants that
+// run without a GPU and the documented corner cases of init_buffer / reshape / assgin.
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <vector>
+
+#include "mini_test.h"
+#include "tensor/tensor.h"
+#include "utils.h"
+
+using namespace base;
+
+template <typename Alloc>
+static void check_shape_api(Alloc allocator, DeviceType where) {
+    {
+        tensor::Tensor t(DataType::DataTypeFp32, 32, true, allocator);
+        ASSERT_EQ(t.is_empty(), false);
+        ASSERT_EQ(t.get_dim(0), 32);
+        ASSERT_EQ(t.size(), 32u);
+        ASSERT_EQ(t.dims(), std::vector<int32_t>({32}));
+        ASSERT_EQ(t.dims_size(), 1);
+        ASSERT_TRUE(t.data_type() == DataType::DataTypeFp32);
+        ASSERT_EQ(t.strides(), std::vector<size_t>({1}));
+        ASSERT_TRUE(t.device_type() == where);
+        ASSERT_EQ(t.byte_size(), 32 * data_type_size(DataType::DataTypeFp32));
+    }
+    {
+        tensor::Tensor t(DataType::DataTypeFp32, 32, 32, true, allocator);
+        ASSERT_EQ(t.get_dim(0), 32);
+        ASSERT_EQ(t.get_dim(1), 32);
+        ASSERT_EQ(t.size(), size_t(32 * 32));
+        ASSERT_EQ(t.dims(), std::vector<int32_t>({32, 32}));
+        ASSERT_EQ(t.dims_size(), 2);
+        ASSERT_EQ(t.strides(), std::vector<size_t>({32, 1}));
+        ASSERT_TRUE(t.device_type() == where);
+        ASSERT_EQ(t.byte_size(), 32 * 32 * sizeof(float));
+    }
+    {
+        tensor::Tensor t(DataType::DataTypeFp32, 12, 22, 32, true, allocator);
+        ASSERT_EQ(t.get_dim(2), 32);
+        ASSERT_EQ(t.size(), size_t(12 * 22 * 32));
+        ASSERT_EQ(t.dims(), std::vector<int32_t>({12, 22, 32}));
+        ASSERT_EQ(t.dims_size(), 3);
+        ASSERT_EQ(t.strides(), std::vector<size_t>({22 * 32, 32, 1}));
+        ASSERT_EQ(t.byte_size(), 12 * 22 * 32 * sizeof(float));
+    }
+    {
+        tensor::Tensor t(DataType::DataTypeFp32, 12, 22, 32, 42, true, allocator);
+        ASSERT_EQ(t.get_dim(3), 42);
+        ASSERT_EQ(t.size(), size_t(12 * 22 * 32 * 42));
+        ASSERT_EQ(t.dims(), std::vector<int32_t>({12, 22, 32, 42}));
+        ASSERT_EQ(t.dims_size(), 4);
+        ASSERT_EQ(t.strides(), std::vector<size_t>({22 * 32 * 42, 32 * 42, 42, 1}));
+        ASSERT_EQ(t.byte_size(), 12 * 22 * 32 * 42 * sizeof(float));
+    }
+    {
+        tensor::Tensor t(DataType::DataTypeFp32, std::vector<int32_t>{12, 22, 32, 42, 52}, true, allocator);
+        ASSERT_EQ(t.is_empty(), false);
+        ASSERT_EQ(t.get_dim(4), 52);
+        ASSERT_EQ(t.size(), size_t(12) * 22 * 32 * 42 * 52);
+        ASSERT_EQ(t.dims(), std::vector<int32_t>({12, 22, 32, 42, 52}));
+        ASSERT_EQ(t.dims_size(), 5);
+        ASSERT_EQ(t.strides(), std::vector<size_t>({22 * 32 * 42 * 52, 32 * 42 * 52, 42 * 52, 52, 1}));
+        ASSERT_TRUE(t.device_type() == where);
+        ASSERT_EQ(t.byte_size(), size_t(12) * 22 * 32 * 42 * 52 * sizeof(float));
+    }
+}
+
+TEST_GPU(test_tensor, init1_to_init5_cuda) {
+    check_shape_api(CUDADeviceAllocatorFactory::get_instance(), DeviceType::DeviceCUDA);
+}
+
+TEST_CPU(test_tensor, init1_to_init5_cpu) {
+    check_shape_api(CPUDeviceAllocatorFactory::get_instance(), DeviceType::DeviceCPU);
+}
+
+TEST_GPU(test_tensor, tensor_base) {
+    auto allocator_cu = CUDADeviceAllocatorFactory::get_instance();
+    tensor::Tensor t_cu(DataType::DataTypeFp32, 32, 32, true, allocator_cu);
+    set_value_cu(t_cu.ptr<float>(), static_cast<int32_t>(t_cu.size()), 1.f);
+    t_cu.to_cpu();
+    ASSERT_TRUE(t_cu.device_type() == DeviceType::DeviceCPU);
+    const float* p = t_cu.ptr<float>();
+    for (size_t i = 0; i < t_cu.size(); i++) ASSERT_EQ(p[i], 1.f);
+    t_cu.to_cpu();  // already there: only logged
+    ASSERT_TRUE(t_cu.device_type() == DeviceType::DeviceCPU);
+}
+
+TEST_GPU(test_tensor, clone_cuda) {
+    auto allocator_cu = CUDADeviceAllocatorFactory::get_instance();
+    tensor::Tensor t1_cu(DataType::DataTypeFp32, 32, 32, true, allocator_cu);
+    set_value_cu(t1_cu.ptr<float>(), static_cast<int32_t>(t1_cu.size()), 1.f);
+    tensor::Tensor t2_cu = t1_cu.clone();
+    ASSERT_EQ(t2_cu.is_empty(), false);
+    ASSERT_EQ(t2_cu.ptr<void>(), t2_cu.get_buffer()->ptr());
+    ASSERT_NE(t2_cu.ptr<void>(), t1_cu.ptr<void>());
+    ASSERT_EQ(t2_cu.dims(), std::vector<int32_t>({32, 32}));
+    ASSERT_EQ(t2_cu.strides(), std::vector<size_t>({32, 1}));
+    ASSERT_TRUE(t2_cu.data_type() == DataType::DataTypeFp32);
+    ASSERT_TRUE(t2_cu.device_type() == DeviceType::DeviceCUDA);
+    ASSERT_EQ(t2_cu.byte_size(), 32 * 32 * sizeof(float));
+    std::vector<float> back(32 * 32, 0.f);
+    allocator_cu->memcpy(back.data(), t2_cu.ptr<float>(), back.size() * sizeof(float), MemcpyKind::MemcpyCUDA2CPU);
+    for (float v : back) ASSERT_EQ(v, 1.f);
+    allocator_cu->memcpy(back.data(), t1_cu.ptr<float>(), back.size() * sizeof(float), MemcpyKind::MemcpyCUDA2CPU);
+    for (float v : back) ASSERT_EQ(v, 1.f);
+    t2_cu.to_cpu();
+    for (size_t i = 0; i < t2_cu.size(); i++) ASSERT_EQ(t2_cu.ptr<float>()[i], 1.f);
+}
+
+TEST_CPU(test_tensor, clone_cpu) {
+    auto allocator = CPUDeviceAllocatorFactory::get_instance();
+    tensor::Tensor t1(DataType::DataTypeFp32, 32, 32, true, allocator);
+    for (size_t i = 0; i < t1.size(); i++) t1.index<float>(i) = 1.f;
+    tensor::Tensor t2 = t1.clone();
+    ASSERT_NE(t2.ptr<void>(), t1.ptr<void>());
+    for (size_t i = 0; i < t2.size(); i++) ASSERT_EQ(t2.ptr<float>()[i], 1.f);
+    t2.index<float>(5) = 9.f;  // deep copy: the source is untouched
+    ASSERT_EQ(t1.index<float>(5), 1.f);
+}
+
+TEST_GPU(test_tensor, to_cuda) {
+    auto allocator_cpu = CPUDeviceAllocatorFactory::get_instance();
+    tensor::Tensor t(DataType::DataTypeFp32, 32, 32, true, allocator_cpu);
+    for (size_t i = 0; i < t.size(); i++) t.ptr<float>()[i] = 1.f;
+    t.to_cuda();
+    ASSERT_TRUE(t.device_type() == DeviceType::DeviceCUDA);
+    std::vector<float> back(32 * 32, 0.f);
+    allocator_cpu->memcpy(back.data(), t.ptr<float>(), back.size() * sizeof(float), MemcpyKind::MemcpyCUDA2CPU);
+    for (float v : back) ASSERT_EQ(v, 1.f);
+}
+
+TEST_CPU(test_tensor, init6_external_pointer) {
+    std::vector<float> storage(32, 0.f);
+    storage[0] = 31;
+    storage[1] = 32;
+    tensor::Tensor t(DataType::DataTypeFp32, 32, false, nullptr, storage.data());
+    ASSERT_TRUE(t.device_type() == DeviceType::DeviceUnknown);
+    t.set_device_type(DeviceType::DeviceCPU);  // const method, writes through to the shared buffer
+    ASSERT_EQ(t.is_empty(), false);
+    ASSERT_EQ(t.get_dim(0), 32);
+    ASSERT_EQ(t.size(), 32u);
+    ASSERT_EQ(t.dims_size(), 1);
+    ASSERT_EQ(t.strides(), std::vector<size_t>({1}));
+    ASSERT_TRUE(t.device_type() == DeviceType::DeviceCPU);
+    ASSERT_EQ(t.byte_size(), 32 * sizeof(float));
+    ASSERT_EQ(t.ptr<float>(), storage.data());
+    ASSERT_EQ(*t.ptr<float>(), 31.f);
+    ASSERT_EQ(*t.ptr<float>(0), 31.f);
+    ASSERT_EQ(*t.ptr<float>(1), 32.f);
+    ASSERT_TRUE(t.get_buffer()->is_external());
+}
+
+TEST_CPU(test_tensor, dims_stride) {
+    auto allocator_cpu = CPUDeviceAllocatorFactory::get_instance();
+    tensor::Tensor t(DataType::DataTypeFp32, 32, 32, 3, true, allocator_cpu);
+    ASSERT_EQ(t.is_empty(), false);
+    const auto& strides = t.strides();
+    ASSERT_EQ(strides.at(0), size_t(32 * 3));
+    ASSERT_EQ(strides.at(1), 3u);
+    ASSERT_EQ(strides.at(2), 1u);
+}
+
+TEST_CPU(test_tensor, assign) {
+    auto allocator_cpu = CPUDeviceAllocatorFactory::get_instance();
+    tensor::Tensor t(DataType::DataTypeFp32, 32, 32, true, allocator_cpu);
+    const size_t size = 32 * 32;
+    std::vector<float> storage(size);
+    for (size_t i = 0; i < size; i++) storage[i] = float(i);
+    auto buffer = std::make_shared<Buffer>(size * sizeof(float), nullptr, storage.data(), true);
+    buffer->set_device_type(DeviceType::DeviceCPU);
+    ASSERT_EQ(t.assgin(buffer), true);
+    ASSERT_EQ(t.is_empty(), false);
+    ASSERT_EQ(t.dims(), std::vector<int32_t>({32, 32}));
+    ASSERT_EQ(t.strides(), std::vector<size_t>({32, 1}));
+    ASSERT_TRUE(t.device_type() == DeviceType::DeviceCPU);
+    ASSERT_EQ(t.ptr<float>(), storage.data());
+    ASSERT_EQ(t.index<float>(77), 77.f);
+    // a too-small buffer is refused, a null one too; the tensor keeps what it had
+    auto small = std::make_shared<Buffer>(16, nullptr, storage.data(), true);
+    ASSERT_EQ(t.assgin(small), false);
+    ASSERT_EQ(t.assgin(nullptr), false);
+    ASSERT_EQ(t.ptr<float>(), storage.data());
+    // a device mismatch is only reported
+    auto other = std::make_shared<Buffer>(size * sizeof(float), nullptr, storage.data(), true);
+    other->set_device_type(DeviceType::DeviceCUDA);
+    ASSERT_EQ(t.assgin(other), true);
+}
+
+TEST_CPU(test_tensor, init_buffer_rules) {
+    auto allocator = CPUDeviceAllocatorFactory::get_instance();
+    // allocator, need_alloc = false, no pointer: allocates all the same
+    tensor::Tensor a(DataType::DataTypeFp32, 8, false, allocator);
+    ASSERT_EQ(a.is_empty(), false);
+    ASSERT_EQ(a.get_buffer()->is_external(), false);
+    // no allocator: a pointer is mandatory and need_alloc must be false
+    ASSERT_FATAL(tensor::Tensor(DataType::DataTypeFp32, 8));
+    std::vector<float> storage(8);
+    ASSERT_FATAL(tensor::Tensor(DataType::DataTypeFp32, 8, true, nullptr, storage.data()));
+    // allocator and pointer: the buffer wraps the pointer and owns it
+    void* mem = allocator->allocate(8 * sizeof(float));
+    {
+        tensor::Tensor owned(DataType::DataTypeFp32, 8, false, allocator, mem);
+        ASSERT_EQ(owned.ptr<void>(), mem);
+        ASSERT_EQ(owned.get_buffer()->is_external(), false);
+        ASSERT_TRUE(owned.device_type() == DeviceType::DeviceUnknown);
+    }
+    // empty dims: zero elements, nothing to allocate
+    tensor::Tensor none(DataType::DataTypeFp32, std::vector<int32_t>{}, true, allocator);
+    ASSERT_EQ(none.size(), 0u);
+    ASSERT_EQ(none.is_empty(), true);
+    ASSERT_EQ(none.strides().size(), 0u);
+    tensor::Tensor blank;
+    ASSERT_EQ(blank.is_empty(), true);
+    ASSERT_EQ(blank.ptr<float>(), nullptr);
+    ASSERT_TRUE(blank.device_type() == DeviceType::DeviceUnknown);
+    ASSERT_FATAL(blank.ptr<float>(0));
+}
+
+TEST_CPU(test_tensor, reshape_reset_index_and_new_element_types) {
+    auto allocator = CPUDeviceAllocatorFactory::get_instance();
+    tensor::Tensor t(DataType::DataTypeFp32, 4, 4, true, allocator);
+    for (int i = 0; i < 16; i++) t.index<float>(i) = float(i);
+    const void* before = t.ptr<void>();
+    t.reshape({2, 8});  // same element count: same storage
+    ASSERT_EQ(t.ptr<void>(), before);
+    ASSERT_EQ(t.dims(), std::vector<int32_t>({2, 8}));
+    t.reshape({2, 4});  // smaller: same storage
+    ASSERT_EQ(t.ptr<void>(), before);
+    ASSERT_EQ(t.size(), 8u);
+    t.reshape({4, 8});  // larger than the current element count: new storage, old contents kept
+    ASSERT_EQ(t.size(), 32u);
+    for (int i = 0; i < 8; i++) ASSERT_EQ(t.index<float>(i), float(i));
+    ASSERT_FATAL(t.index<float>(32));
+    ASSERT_FATAL(t.index<float>(-1));
+    ASSERT_FATAL(t.get_dim(2));
+    t.reset(DataType::DataTypeInt32, {3, 5});
+    ASSERT_EQ(t.is_empty(), true);
+    ASSERT_EQ(t.size(), 15u);
+    ASSERT_EQ(t.get_buffer(), nullptr);
+    ASSERT_EQ(t.allocate(nullptr, false), false);
+    ASSERT_EQ(t.allocate(allocator, false), true);
+    ASSERT_EQ(t.byte_size(), 15 * sizeof(int32_t));
+    // element types added for the matmul path
+    ASSERT_EQ(data_type_size(DataType::DataTypeBf16), 2u);
+    ASSERT_EQ(data_type_size(DataType::DataTypeFp16), 2u);
+    ASSERT_EQ(data_type_size(DataType::DataTypeInt8), 1u);
+    ASSERT_FATAL(data_type_size(DataType::DataTypeUnknown));
+    tensor::Tensor h(DataType::DataTypeBf16, 3, 128, true, allocator);
+    ASSERT_EQ(h.byte_size(), size_t(3 * 128 * 2));
+    // values of the pre-existing members are unchanged
+    ASSERT_EQ(int(DataType::DataTypeFp32), 1);
+    ASSERT_EQ(int(DataType::DataTypeInt8), 2);
+    ASSERT_EQ(int(DataType::DataTypeInt32), 3);
+    ASSERT_EQ(int(DeviceType::DeviceCUDA), 2);
+}
