@@ -28,9 +28,10 @@ HBM_PEAK_GBPS = 8000.0
 WEIGHT_SETS = 12           # x 100.4 MB per set = 1.2 GB of cold weights
 ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
 METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until such a run has been made for the current kernel.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the dominant kernel (average over the seven launches of a step) from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
+# reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).
+TRAFFIC_BYTES_PER_LAUNCH = 15374000
 
 
 def parse_args():
@@ -42,6 +43,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-passes", type=int, default=30)
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter-collection workload: one 256 MiB device copy (known traffic, for scaling the "
+                         "counters) followed by a few cold launches per projection shape; prints no metric")
     return ap.parse_args()
 
 
@@ -151,6 +155,16 @@ def main():
             for n in ORDER:
                 qw, sc, qz = wset.t[n]
                 capi.gemv_awq_bf16(xs[shapes[n][0]], qw, sc, qz, ys[n], group, ws)
+
+    if args.probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        launch_steps(0, WEIGHT_SETS)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy 268435456 B, then %d steps of 7 launches" % WEIGHT_SETS}))
+        return
 
     seconds = timed_region(torch, launch_steps, args.steps, args.warmup, args.eager, WEIGHT_SETS)
     ms_per_step = seconds / args.steps * 1e3
