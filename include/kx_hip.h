@@ -78,6 +78,13 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
                      const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
                      int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Two kernels implement kx_gemv_awq_bf16: one on the vector ALUs (used for M = 1) and one on the
+ * matrix cores (MFMA; used for M >= 2 when the group size is a power of two).  This knob overrides
+ * the choice for tuning and for tests: 0 = by shape (default), 1 = always the vector kernel,
+ * 2 = the MFMA kernel wherever the group size allows.  Process-wide, not thread-safe.
+ * Reference counterpart: none. */
+int kx_set_awq_kernel_policy(int policy);
+
 /* ------------------------------------------------------------------------------------------
  * BF16 GEMV fallback (non-quantised layers, lm_head):   y[m,n] = sum_k x[m,k] * W[n,k]
  *   W bf16 [N,K] row-major (dim0 = output features, dim1 = input features, the reading of

@@ -21,6 +21,7 @@ SIGNATURES = {
     "kx_gemv_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kx_workspace_init": (ctypes.c_int, [_P, _SZ, _P]),
     "kx_gemv_awq_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_set_awq_kernel_policy": (ctypes.c_int, [ctypes.c_int]),
     "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
@@ -91,6 +92,11 @@ def gemv_awq_bf16(x, qweight, scales, qzeros, y, group_size, workspace):
     _check(load().kx_gemv_awq_bf16(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
                                    M, K, N, group_size, _ptr(workspace),
                                    0 if workspace is None else workspace.numel(), _stream()))
+
+
+def set_awq_kernel_policy(policy):
+    """0 = choose by shape, 1 = vector-ALU kernel, 2 = MFMA kernel where the group size allows."""
+    _check(load().kx_set_awq_kernel_policy(policy))
 
 
 def gemv_bf16(x, w, y, workspace=None):

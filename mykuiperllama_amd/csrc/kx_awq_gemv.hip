@@ -1,12 +1,15 @@
 // Host side of the fused INT4 AWQ dequantise + GEMV: shape checks, launch plan, C ABI.
 #include "kx_awq_gemv_kernel.h"
+#include "kx_awq_gemv_mfma_kernel.h"
+
 
 namespace kx {
 namespace {
 
 struct AwqPlan {
+    bool mfma;     // matrix-core kernel (any M) or the VALU kernel
     int waves;     // waves per workgroup stacked along K (4, 8 or 16)
-    int rt;        // consecutive rows per lane (8 or 16)
+    int rt;        // VALU kernel: consecutive rows per lane (8 or 16); MFMA kernel: 32-row steps per wave
     int mb;        // activation rows per workgroup (1, 2, 4 or 8)
     int coltiles;  // tiles of 256 output columns
     int ktiles;    // workgroups along K that share a column tile
@@ -17,11 +20,43 @@ inline int rows_per_block(int waves, int rt) {
     return waves * kSlotsPerWave * rt;
 }
 
-inline AwqPlan make_plan(int M, int K, int N) {
+// 0: choose by shape; 1: always the VALU kernel; 2: the MFMA kernel wherever the group size allows
+int g_kernel_policy = 0;
+
+inline int kernel_override() {
+    return g_kernel_policy;
+}
+
+inline bool is_pow2(int v) {
+    return v > 0 && (v & (v - 1)) == 0;
+}
+
+// MFMA kernel: four waves per workgroup, each walking `ks` consecutive 32-row steps that must lie in
+// one quantisation group.  Measured on the Qwen3-8B shapes: two steps per wave (256 rows per
+// workgroup) are best for M = 2..4, four steps (512 rows, half the partial sums to exchange) from
+// M = 5 on, where the exchange grows with M.
+inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     AwqPlan p;
+    p.mfma = true;
+    p.coltiles = (N / 8 + kWC - 1) / kWC;
+    p.mb = M;
+    p.mtiles = 1;
+    p.waves = 4;
+    int ks = M >= 5 ? 4 : 2;
+    while (ks > 1 && ks * kStepRows > group) ks /= 2;
+    while (ks > 1 && p.waves * ks * kStepRows > K) ks /= 2;
+    p.rt = ks;  // steps per wave
+    const int kb = p.waves * ks * kStepRows;
+    p.ktiles = (K + kb - 1) / kb;
+    return p;
+}
+
+inline AwqPlan make_valu_plan(int M, int K, int N) {
+    AwqPlan p;
+    p.mfma = false;
+    p.coltiles = (N / 8 + kWC - 1) / kWC;
     p.mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
     p.mtiles = (M + p.mb - 1) / p.mb;
-    p.coltiles = (N / 8 + kWC - 1) / kWC;
     // Eight waves of sixteen rows per lane (256 rows of K per workgroup) measured best or within
     // noise of best on every Qwen3 projection shape; shorter K takes fewer waves so that no
     // workgroup is mostly idle.
@@ -32,6 +67,14 @@ inline AwqPlan make_plan(int M, int K, int N) {
     const int kb = rows_per_block(p.waves, p.rt);
     p.ktiles = (K + kb - 1) / kb;
     return p;
+}
+
+inline AwqPlan make_plan(int M, int K, int N, int group) {
+    // The MFMA kernel needs quantisation groups that tile the workgroup's K range: powers of two.
+    const bool mfma_ok = is_pow2(group);
+    const int mode = kernel_override();
+    const bool mfma = mfma_ok && (mode == 2 || (mode == 0 && M >= 2));
+    return mfma ? make_mfma_plan(M, K, N, group) : make_valu_plan(M, K, N);
 }
 
 template <int WAVES, int RT>
@@ -56,10 +99,19 @@ __global__ void fill_zero_u32(uint32_t* p, size_t n) {
 }  // namespace
 }  // namespace kx
 
+extern "C" int kx_set_awq_kernel_policy(int policy) {
+    if (policy < 0 || policy > 2) return KX_ERR_BAD_SHAPE;
+    kx::g_kernel_policy = policy;
+    return KX_OK;
+}
+
 extern "C" size_t kx_gemv_workspace_bytes(int32_t M, int32_t K, int32_t N) {
     if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8) return 0;
-    const kx::AwqPlan p = kx::make_plan(M, K, N);
-    return kx::kCounterBytes + static_cast<size_t>(p.ktiles) * M * static_cast<size_t>(N) * sizeof(float);
+    // Either kernel may serve a shape (the group size and M decide); size for the larger exchange.
+    const int kt_valu = kx::make_valu_plan(M, K, N).ktiles;
+    const int kt_mfma = kx::make_mfma_plan(M, K, N, 32).ktiles;  // the smallest group gives the most K tiles
+    const size_t ktiles = static_cast<size_t>(kt_valu > kt_mfma ? kt_valu : kt_mfma);
+    return kx::kCounterBytes + ktiles * M * static_cast<size_t>(N) * sizeof(float);
 }
 
 extern "C" int kx_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
@@ -85,7 +137,7 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
         reinterpret_cast<uintptr_t>(y) % 8) {
         return KX_ERR_ALIGNMENT;
     }
-    kx::AwqPlan p = kx::make_plan(M, K, N);
+    kx::AwqPlan p = kx::make_plan(M, K, N, group_size);
     float* partials = nullptr;
     uint32_t* counters = nullptr;
     if (p.ktiles > 1) {
@@ -98,6 +150,24 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
         partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kx::kCounterBytes);
     }
     hipStream_t s = kx::as_stream(stream);
+    if (p.mfma) {
+        int group_shift = 0;
+        while ((1 << group_shift) < group_size) group_shift++;
+#define KX_MARGS x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_shift, p.coltiles, p.ktiles, s
+#define KX_MFMA_BY_M(KS)                                                        \
+    do {                                                                        \
+        if (M == 1) kx::launch_awq_gemv_mfma<4, KS, 1, 1>(KX_MARGS);            \
+        else if (M == 2) kx::launch_awq_gemv_mfma<4, KS, 2, 1>(KX_MARGS);       \
+        else if (M <= 4) kx::launch_awq_gemv_mfma<4, KS, 4, 1>(KX_MARGS);       \
+        else kx::launch_awq_gemv_mfma<4, KS, 4, 4>(KX_MARGS);                   \
+    } while (0)
+        if (p.rt == 4) KX_MFMA_BY_M(4);
+        else if (p.rt == 2) KX_MFMA_BY_M(2);
+        else KX_MFMA_BY_M(1);
+#undef KX_MFMA_BY_M
+#undef KX_MARGS
+        return kx::launch_status();
+    }
 #define KX_ARGS p, x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_size, s
     if (p.waves == 8) {
         kx::launch_mb<8, 16>(KX_ARGS);

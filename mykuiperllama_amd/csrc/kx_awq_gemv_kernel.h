@@ -16,33 +16,22 @@
 // tile column t in that exchange, so every store and load of partials is a contiguous 256 bytes
 // per wave.
 //
-// Cross-XCD visibility without cache-wide fences: partials are stored write-through at device
-// scope and read back with device-scope loads; the counter is a device-scope atomic.  The wave
-// waits for its own stores to be acknowledged before it touches the counter, which is all the
-// ordering the exchange needs.  (A device-scope fence would write back and invalidate the whole
-// L2 once per workgroup; measured at ~0.25 us per workgroup, serialised.)
+// The exchange itself is in kx_splitk_exchange.h.
 #ifndef KX_AWQ_GEMV_KERNEL_H
 #define KX_AWQ_GEMV_KERNEL_H
 
 #include "kx_common.h"
+#include "kx_splitk_exchange.h"
 
 namespace kx {
 
 constexpr int kWC = 32;                 // word columns per wave
-constexpr int kTileCols = kWC * 8;      // output columns per column tile
+static_assert(kWC * 8 == kTileCols, "a wave spans one column tile");
 constexpr int kSlotsPerWave = kWave / kWC;
-constexpr int kCounterStride = 16;      // uint32 slots between counters: one 64-byte line each
 
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ void store_agent(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float load_agent(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // The eight codes of a packed word as floats, indexed by column (0..7) inside the word.
 // A byte 0x0q read as OCP fp8 (e4m3) is exactly q * 2^-9 for every q in 0..15 (subnormal below
@@ -201,65 +190,9 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
     }
 
-    const int col = ct * kTileCols + tid;
-    const bool col_ok = (tid < kTileCols) && (col < N);
-    if (ktiles == 1) {
-        if (col_ok) {
-#pragma unroll
-            for (int m = 0; m < MB; m++) {
-                if (m0 + m < M) y[static_cast<size_t>(m0 + m) * N + col] = f32_to_bf16(psum[m]);
-            }
-        }
-        return;
-    }
-
-    // Exchange between the workgroups of this column tile.
     __shared__ uint32_t s_prev;
-    const size_t tstride = static_cast<size_t>(M) * N;  // floats between consecutive K tiles
-    if (col_ok) {
-#pragma unroll
-        for (int m = 0; m < MB; m++) {
-            if (m0 + m < M) {
-                store_agent(partials + static_cast<size_t>(kt) * tstride + static_cast<size_t>(m0 + m) * N + col, psum[m]);
-            }
-        }
-    }
-    // every wave waits until its stores have been acknowledged (no cache-wide action), then the
-    // barrier orders all of them before the counter moves
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    uint32_t* counter = counters + static_cast<size_t>(blockIdx.y * coltiles + ct) * kCounterStride;
-    if (tid == 0) {
-        s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (s_prev != static_cast<uint32_t>(ktiles - 1)) return;
-
-    // Last to arrive: every other workgroup's partials were acknowledged before its increment.
-    if (col_ok) {
-#pragma unroll
-        for (int m = 0; m < MB; m++) {
-            if (m0 + m >= M) break;
-            const float* pp = partials + static_cast<size_t>(m0 + m) * N + col;
-            float sum = 0.0f;
-            // sixteen loads in flight at a time; the additions keep the order t = 0, 1, 2, ...
-            for (int t0 = 0; t0 < ktiles; t0 += 16) {
-                float v[16];
-#pragma unroll
-                for (int u = 0; u < 16; u++) {
-                    v[u] = (t0 + u < ktiles) ? load_agent(pp + static_cast<size_t>(t0 + u) * tstride) : 0.0f;
-                }
-#pragma unroll
-                for (int u = 0; u < 16; u++) sum += v[u];
-            }
-            y[static_cast<size_t>(m0 + m) * N + col] = f32_to_bf16(sum);
-        }
-    }
-    if (tid == 0) {
-        // leave the workspace ready for the next launch
-        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
+                              &s_prev);
 }
 
 template <int WAVES, int RT, int MB>

@@ -1,0 +1,250 @@
+// Fused INT4 AWQ dequantise + GEMV on the matrix cores (gfx950, v_mfma_f32_16x16x32_bf16), M <= 16.
+//
+//   y[m,n] = sum_k x[m,k] * (q[k,n] - z[k/G,n]) * s[k/G,n]
+//
+// One MFMA multiplies A = activations (16 rows m x 32 k) by B = weights (32 k x 16 columns n) into a
+// 16 x 16 fp32 tile.  Lane l of the wave supplies, for both operands, the eight k values
+// 8*(l/16) .. 8*(l/16)+7 of row / column l%16, and receives D[4*(l/16)+v][l%16], v = 0..3.
+//
+// A lane (c = l%16, b = l/16) loads the two packed words (c-th pair of the tile's 32 word columns)
+// of the eight rows 8b .. 8b+7 of a 32-row step: sixteen columns x eight rows of codes.  Nibble p of
+// word h of those eight rows is exactly the B operand of column 8*(2c+h) + ORDER[p], so sixteen
+// MFMAs per step - one per (h, p) - cover the lane's sixteen columns, all with the same A operand,
+// which is a plain 16-byte load of x.  A code becomes a bf16 by OR-ing it into the mantissa of
+// 128.0 (0x4300 | q = 128 + q, exact), two rows per register; the +128 joins the zero point:
+//
+//   sum_k x*(q - z) = sum_k x*(128 + q)  -  (128 + z) * sum_k x
+//
+// and sum_k x comes out of one more MFMA against a B operand of ones, in the same register layout.
+// Raw sums of the waves of a workgroup meet in LDS; the thread that owns a column applies zero
+// point and scale once per wave (a wave never straddles a quantisation group: groups are powers of
+// two here and the host picks KS so that KS*32 divides the group) and takes part in the split-K exchange.
+//
+// Cost per weight: one VALU operation to build the operand (two byte permutes, three shifts and
+// eight and/or pairs per sixteen weights) and 1/512 of an MFMA, whatever M is.
+#ifndef KX_AWQ_GEMV_MFMA_KERNEL_H
+#define KX_AWQ_GEMV_MFMA_KERNEL_H
+
+#include "kx_common.h"
+#include "kx_splitk_exchange.h"
+
+namespace kx {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+constexpr int kStepRows = 32;  // rows of K per MFMA step
+
+// Column (0..7) inside a word -> nibble that holds it (inverse of order_of).
+__host__ __device__ constexpr int nibble_of(int col) {
+    return (col & 1) ? 4 + (col >> 1) : (col >> 1);
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    u32x4 v = {a, b, c, d};
+    bf16x8 out;
+    __builtin_memcpy(&out, &v, 16);
+    return out;
+}
+
+// Two bf16 128.0 in a register whose value the compiler cannot see.  (v & 0x000F000F) | magic then
+// selects as one v_and_or_b32 (a literal and a register); with two literals it would be split into
+// v_and + v_or.  The conversion itself stays ordinary C so that the compiler keeps track of the
+// registers the matrix instructions are still reading.
+__device__ __forceinline__ uint32_t opaque_bf16_128_pair() {
+    uint32_t out;
+    asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(out));
+    return out;
+}
+
+__device__ __forceinline__ uint32_t code_pair_to_bf16(uint32_t v, uint32_t magic) {
+    return (v & 0x000F000Fu) | magic;
+}
+
+// KS: consecutive 32-row steps per wave (they must share a quantisation group);
+// MC: activation rows a workgroup reduces per LDS round (1, 2 or 4); ROUNDS: 1 for M <= 4, else 4.
+template <int WAVES, int KS, int MC, int ROUNDS>
+__global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
+    uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
+    int M, int K, int N, int group_shift, int ktiles) {
+    constexpr int WROWS = KS * kStepRows;  // rows of K per wave
+    constexpr int KB = WAVES * WROWS;      // rows of K per workgroup
+    constexpr int ROWS = MC * ROUNDS;      // activation rows this kernel carries (>= M)
+    static_assert(WAVES * kWave >= kTileCols, "one thread per tile column");
+
+    __shared__ __attribute__((aligned(16))) float red[WAVES][MC][kTileCols];
+    __shared__ float xs_red[WAVES][MC];
+    __shared__ uint32_t s_prev;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int c = lane % 16;  // column slot: word pair c of the tile, MFMA column c
+    const int b = lane / 16;  // k block inside the step, D row block
+    const int ct = blockIdx.x;  // column tile; x runs fastest, so neighbours in time are neighbours in N
+    const int kt = blockIdx.y;
+    const int nw = N >> 3;
+
+    const int wcg = ct * 32 + 2 * c;           // first of the lane's two word columns
+    const int kwave = kt * KB + wave * WROWS;  // first row of this wave
+    const bool w0_ok = wcg < nw;
+    const bool w1_ok = wcg + 1 < nw;
+
+    // ---- loads, all issued before anything is consumed ----
+    // Scale and zero point of the column this thread will own after the LDS round, one pair per
+    // wave of the workgroup (a wave never straddles a quantisation group; waves that share a group
+    // read the same address).  Everything below is indexed at compile time.
+    const int own_col = ct * kTileCols + tid;
+    const bool own_ok = (tid < kTileCols) && (own_col < N);
+    uint16_t s_bits[WAVES];
+    uint32_t z_word[WAVES];
+#pragma unroll
+    for (int wv = 0; wv < WAVES; wv++) {
+        const int krow = kt * KB + wv * WROWS;
+        const bool ok = own_ok && krow < K;
+        const int g = krow >> group_shift;
+        s_bits[wv] = ok ? scales[static_cast<size_t>(g) * N + own_col] : static_cast<uint16_t>(0);
+        z_word[wv] = ok ? qzeros[static_cast<size_t>(g) * nw + (own_col >> 3)] : 0u;
+    }
+    uint4 xa[KS];
+    uint32_t w[KS][8][2];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        xa[ks] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int r = 0; r < 8; r++) w[ks][r][0] = w[ks][r][1] = 0u;
+    }
+    if (c < M) {
+        // the A operand: row c of the activations, whether or not column slot c holds weights
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int kstep = kwave + ks * kStepRows;
+            if (kstep < K) xa[ks] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(c) * K + kstep + 8 * b);
+        }
+    }
+    if (w0_ok) {
+        const bool pair_loads = (nw & 1) == 0;  // rows are 8-byte aligned: both words in one load
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int kstep = kwave + ks * kStepRows;
+            if (kstep < K) {  // K is a multiple of 32: a step is all in or all out (wave-uniform)
+                const int k0 = kstep + 8 * b;  // first of the lane's eight rows
+                const uint32_t* wp = qweight + static_cast<size_t>(k0) * nw + wcg;
+                if (pair_loads) {
+#pragma unroll
+                    for (int r = 0; r < 8; r++) {
+                        const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(wp + static_cast<size_t>(r) * nw));
+                        w[ks][r][0] = v.x;
+                        w[ks][r][1] = v.y;
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 8; r++) {
+                        w[ks][r][0] = __builtin_nontemporal_load(wp + static_cast<size_t>(r) * nw);
+                        if (w1_ok) w[ks][r][1] = __builtin_nontemporal_load(wp + static_cast<size_t>(r) * nw + 1);
+                    }
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- matrix products ----
+    const bf16x8 ones = as_bf16x8(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
+    const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4v xs;
+    f32x4v acc[2][8];  // [word h][nibble p]
+    const uint32_t magic = opaque_bf16_128_pair();
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const bf16x8 a_op = as_bf16x8(xa[ks].x, xa[ks].y, xa[ks].z, xa[ks].w);
+        xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, ones, ks == 0 ? zero4 : xs, 0, 0, 0);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t bop[8][4];  // [nibble p][row pair]
+#pragma unroll
+            for (int rp = 0; rp < 4; rp++) {
+                const uint32_t wa = w[ks][2 * rp][h];      // row 2rp   -> low half
+                const uint32_t wb = w[ks][2 * rp + 1][h];  // row 2rp+1 -> high half
+                const uint32_t lo = __builtin_amdgcn_perm(wb, wa, 0x05040100u);  // nibbles 0..3, both rows
+                const uint32_t hi = __builtin_amdgcn_perm(wb, wa, 0x07060302u);  // nibbles 4..7
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    bop[p][rp] = code_pair_to_bf16(p == 0 ? lo : lo >> (4 * p), magic);
+                    bop[4 + p][rp] = code_pair_to_bf16(p == 0 ? hi : hi >> (4 * p), magic);
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < 8; p++) {
+                acc[h][p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    a_op, as_bf16x8(bop[p][0], bop[p][1], bop[p][2], bop[p][3]), ks == 0 ? zero4 : acc[h][p], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- waves meet in LDS; thread t < 256 then owns tile column t ----
+    float psum[ROWS];
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; rd++) {
+        if (rd > 0) __syncthreads();  // the previous round has been read
+        if (b == rd) {
+            // D rows 4b + v are activation rows 4*rd + v; the lane's sixteen columns are 16c .. 16c+15
+#pragma unroll
+            for (int v = 0; v < MC; v++) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    f32x4* dst = reinterpret_cast<f32x4*>(&red[wave][v][16 * c + 8 * h]);
+                    dst[0] = f32x4{acc[h][nibble_of(0)][v], acc[h][nibble_of(1)][v], acc[h][nibble_of(2)][v],
+                                   acc[h][nibble_of(3)][v]};
+                    dst[1] = f32x4{acc[h][nibble_of(4)][v], acc[h][nibble_of(5)][v], acc[h][nibble_of(6)][v],
+                                   acc[h][nibble_of(7)][v]};
+                }
+                if (c == 0) xs_red[wave][v] = xs[v];
+            }
+        }
+        __syncthreads();
+        if (tid < kTileCols) {
+            float qv[MC][WAVES], xv[MC][WAVES];
+#pragma unroll
+            for (int v = 0; v < MC; v++) {
+#pragma unroll
+                for (int wv = 0; wv < WAVES; wv++) {
+                    qv[v][wv] = red[wv][v][tid];
+                    xv[v][wv] = xs_red[wv][v];
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < MC; v++) {
+                float total = 0.0f;
+#pragma unroll
+                for (int wv = 0; wv < WAVES; wv++) {
+                    const float s = f16_bits_to_f32(s_bits[wv]);
+                    const float z = static_cast<float>((z_word[wv] >> (4 * nibble_of(own_col & 7))) & 0xFu);
+                    total += s * __builtin_fmaf(-(128.0f + z), xv[v][wv], qv[v][wv]);
+                }
+                psum[rd * MC + v] = total;
+            }
+        }
+    }
+
+    splitk_exchange_store<ROWS>(psum, 0, M, N, ct, kt, ktiles, ct, partials, counters, y, &s_prev);
+}
+
+template <int WAVES, int KS, int MC, int ROUNDS>
+inline void launch_awq_gemv_mfma(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
+                                 const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
+                                 int M, int K, int N, int group_shift, int coltiles, int ktiles,
+                                 hipStream_t stream) {
+    dim3 grid(coltiles, ktiles, 1);
+    dim3 block(WAVES * kWave, 1, 1);
+    hipLaunchKernelGGL((awq_gemv_mfma_kernel<WAVES, KS, MC, ROUNDS>), grid, block, 0, stream, x,
+                       reinterpret_cast<const uint32_t*>(qweight), scales,
+                       reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
+                       group_shift, ktiles);
+}
+
+}  // namespace kx
+
+#endif  // KX_AWQ_GEMV_MFMA_KERNEL_H

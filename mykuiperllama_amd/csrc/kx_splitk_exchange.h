@@ -1,0 +1,108 @@
+// Split-K exchange shared by the GEMV kernels: the workgroups that cover different K ranges of one
+// 256-column tile meet in a caller-provided workspace and the one that arrives last finishes the
+// sum in a fixed order (bitwise reproducible) and writes the bf16 output.
+//
+// Cross-XCD visibility without cache-wide fences: partials are stored write-through at device
+// scope and read back with device-scope loads; the counter is a device-scope atomic.  Every wave
+// waits for its own stores to be acknowledged before the barrier, and the counter moves after the
+// barrier: that is all the ordering the exchange needs.  (A device-scope fence would write back and
+// invalidate the whole L2 once per workgroup: measured ~0.25 us per workgroup, serialised.)
+// Counters sit on 64-byte lines of their own; packed together they serialise at the memory side
+// (~10 ns per atomic, measured).
+#ifndef KX_SPLITK_EXCHANGE_H
+#define KX_SPLITK_EXCHANGE_H
+
+#include "kx_common.h"
+
+namespace kx {
+
+constexpr int kTileCols = 256;     // output columns per column tile, one thread each in the exchange
+constexpr int kCounterStride = 16; // uint32 slots between counters: one 64-byte line each
+
+__device__ __forceinline__ void store_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Called by every thread of the workgroup (it contains barriers).  Thread tid < 256 owns tile column
+// tid and brings psum[r], its partial sum for activation row m0 + r.  `s_prev` is one uint32 of LDS.
+template <int ROWS>
+__device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS], int m0, int M, int N,
+                                                      int ct, int kt, int ktiles, int counter_index,
+                                                      float* __restrict__ partials,
+                                                      uint32_t* __restrict__ counters,
+                                                      uint16_t* __restrict__ y, uint32_t* s_prev) {
+    const int tid = threadIdx.x;
+    const int col = ct * kTileCols + tid;
+    const bool col_ok = (tid < kTileCols) && (col < N);
+    if (ktiles == 1) {
+        if (col_ok) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(psum[r]);
+            }
+        }
+        return;
+    }
+
+    const size_t tstride = static_cast<size_t>(M) * N;  // floats between consecutive K tiles
+    if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            if (m0 + r < M) {
+                store_agent(partials + static_cast<size_t>(kt) * tstride + static_cast<size_t>(m0 + r) * N + col, psum[r]);
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    uint32_t* counter = counters + static_cast<size_t>(counter_index) * kCounterStride;
+    if (tid == 0) {
+        *s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return;
+
+    // Last to arrive: every other workgroup's partials were acknowledged before its increment.
+    // Up to 64 loads are in flight per thread (TB K-tiles of every row at a time); per row the
+    // additions keep the order t = 0, 1, 2, ...
+    if (col_ok) {
+        constexpr int TB = ROWS >= 16 ? 4 : 16;
+        float sum[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) sum[r] = 0.0f;
+        const float* pp = partials + col;
+        for (int t0 = 0; t0 < ktiles; t0 += TB) {
+            float v[ROWS][TB];
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+#pragma unroll
+                for (int u = 0; u < TB; u++) {
+                    v[r][u] = (m0 + r < M && t0 + u < ktiles)
+                        ? load_agent(pp + static_cast<size_t>(t0 + u) * tstride + static_cast<size_t>(m0 + r) * N)
+                        : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+#pragma unroll
+                for (int u = 0; u < TB; u++) sum[r] += v[r][u];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(sum[r]);
+        }
+    }
+    if (tid == 0) {
+        // leave the workspace ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+}  // namespace kx
+
+#endif  // KX_SPLITK_EXCHANGE_H

@@ -59,6 +59,14 @@ def check_against_oracle(oracle, p, y_bits):
 SHAPES_8B = sorted(set(synth.QWEN3_8B.values()))
 
 
+@pytest.fixture(params=["by_shape", "vector", "mfma"], autouse=True)
+def kernel_policy(request, capi):
+    """Every test in this file runs under all three kernel policies."""
+    capi.set_awq_kernel_policy({"by_shape": 0, "vector": 1, "mfma": 2}[request.param])
+    yield request.param
+    capi.set_awq_kernel_policy(0)
+
+
 @pytest.mark.parametrize("K,N", [(1024, 2048)] + SHAPES_8B)
 def test_gemv_m1_matches_oracle(capi, torch, oracle, K, N):
     p = synth.make_awq_problem(f"gemv_m1_{K}x{N}", 1, K, N)
@@ -119,7 +127,7 @@ def test_repeated_launches_are_bitwise_identical_and_workspace_reusable(capi, to
 
 
 @pytest.mark.parametrize("K,N,G", [(128, 8, 128), (256, 24, 128), (384, 264, 128), (64, 2056, 32),
-                                   (2048, 40, 64)])
+                                   (2048, 40, 64), (1024, 512, 256), (1024, 1000, 512), (192, 64, 96)])
 def test_ragged_and_small_shapes(capi, torch, oracle, K, N, G):
     p = synth.make_awq_problem(f"ragged_{K}x{N}", 3, K, N, group=G)
     y, _ = run_awq(capi, torch, p)
