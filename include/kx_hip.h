@@ -110,6 +110,47 @@ int kx_awq_unpack_u8(const int32_t* words, uint8_t* codes, int64_t rows, int64_t
 int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
                         uint16_t* w, int32_t K, int32_t N, int32_t group_size, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Supporting kernels of a Qwen3-style decode step, batch 1 (bf16 storage, fp32 arithmetic).
+ * The reference reserves the layer slots (LayerRMSNorm, LayerRope, LayerMHA, LayerSwiGLU, LayerAdd,
+ * LayerEmbedding: kuiper/include/op/layer.h:8-20) and leaves the operators empty
+ * (kuiper/include/op/{rmsnorm,rope,mha,swiglu,embedding}.h); these are the GPU kernels a
+ * get_*_kernel(DeviceCUDA) entry for them would return.  All pointers 16-byte aligned unless noted.
+ *
+ *   kx_rmsnorm_bf16       y[r,:] = gain * bf16(x[r,:] * rsqrt(mean(x[r,:]^2) + eps)),  n % 8 == 0
+ *   kx_add_rmsnorm_bf16   x <- bf16(x + delta) in place (the residual add), then as above on the new x
+ *   kx_qk_norm_rope_bf16  qkv = [q heads | k heads | v heads] x 128: RMSNorm over each q / k head with
+ *                         its 128-element gain, rotary embedding at *pos (rotate-half convention,
+ *                         frequencies theta^(-i/64)), q to q_out, k and v to row *pos of the caches
+ *                         (bf16 [max_positions][n_kv_heads][128]).  head_dim must be 128.
+ *   kx_attn_decode_bf16   GQA attention of one query position against cache rows 0 .. *pos:
+ *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv in
+ *                         {1,2,4,8}; split over the context in chunks of 128 positions, merged by
+ *                         log-sum-exp.  `max_positions` fixes the launch shape (a captured graph can be
+ *                         replayed while *pos advances up to max_positions - 1).
+ *   kx_swiglu_bf16        out = bf16(silu(gate)) * up
+ *   kx_add_bf16           out = a + b   (the reference's add operator, add_kernel.cu:4-12, in bf16)
+ *   kx_embedding_bf16     out = table[*token, :]   (token clamped to the vocabulary)
+ *   kx_argmax_bf16        *out_index = first index of the largest value (NaN ignored)
+ * `pos` and `token` are DEVICE pointers to one int32, so that a captured graph sees new values.
+ * ------------------------------------------------------------------------------------------ */
+int kx_rmsnorm_bf16(const uint16_t* x, const uint16_t* gain, uint16_t* y, int32_t rows, int32_t n, float eps,
+                    void* stream);
+int kx_add_rmsnorm_bf16(uint16_t* x_inout, const uint16_t* delta, const uint16_t* gain, uint16_t* y,
+                        int32_t rows, int32_t n, float eps, void* stream);
+int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain, uint16_t* q_out,
+                         uint16_t* k_cache, uint16_t* v_cache, int32_t n_q_heads, int32_t n_kv_heads,
+                         int32_t head_dim, const int32_t* pos, float rope_theta, float eps, void* stream);
+size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head_dim, int32_t max_positions);
+int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, uint16_t* out,
+                        int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
+                        int32_t max_positions, void* workspace, size_t workspace_bytes, void* stream);
+int kx_swiglu_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int32_t n, void* stream);
+int kx_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int32_t n, void* stream);
+int kx_embedding_bf16(const uint16_t* table, const int32_t* token, uint16_t* out, int32_t vocab, int32_t dim,
+                      void* stream);
+int kx_argmax_bf16(const uint16_t* x, int32_t n, int32_t* out_index, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,16 @@ SIGNATURES = {
     "kx_set_awq_kernel_policy": (ctypes.c_int, [ctypes.c_int]),
     "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
+    "kx_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
+    "kx_add_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
+    "kx_qk_norm_rope_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, ctypes.c_float,
+                                            ctypes.c_float, _P]),
+    "kx_attn_decode_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "kx_attn_decode_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _SZ, _P]),
+    "kx_swiglu_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _P]),
+    "kx_add_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _P]),
+    "kx_embedding_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _P]),
+    "kx_argmax_bf16": (ctypes.c_int, [_P, _I32, _P, _P]),
     "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
 }
 
@@ -116,3 +126,47 @@ def awq_dequant_bf16(qweight, scales, qzeros, w, group_size):
     K, wcols = qweight.shape
     _check(load().kx_awq_dequant_bf16(_ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(w), K,
                                       wcols * 8, group_size, _stream()))
+
+
+# ---------------------------------------------------------------- decode-step operators
+def rmsnorm_bf16(x, gain, y, eps):
+    rows = x.numel() // x.shape[-1]
+    _check(load().kx_rmsnorm_bf16(_ptr(x), _ptr(gain), _ptr(y), rows, x.shape[-1], eps, _stream()))
+
+
+def add_rmsnorm_bf16(x_inout, delta, gain, y, eps):
+    rows = x_inout.numel() // x_inout.shape[-1]
+    _check(load().kx_add_rmsnorm_bf16(_ptr(x_inout), _ptr(delta), _ptr(gain), _ptr(y), rows, x_inout.shape[-1],
+                                      eps, _stream()))
+
+
+def qk_norm_rope_bf16(qkv, q_gain, k_gain, q_out, k_cache, v_cache, n_q, n_kv, pos, theta, eps):
+    _check(load().kx_qk_norm_rope_bf16(_ptr(qkv), _ptr(q_gain), _ptr(k_gain), _ptr(q_out), _ptr(k_cache),
+                                       _ptr(v_cache), n_q, n_kv, 128, _ptr(pos), theta, eps, _stream()))
+
+
+def attn_decode_workspace(n_q, max_positions, device="cuda"):
+    import torch
+    nbytes = int(load().kx_attn_decode_workspace_bytes(n_q, 128, max_positions))
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def attn_decode_bf16(q, k_cache, v_cache, out, n_q, n_kv, pos, max_positions, workspace):
+    _check(load().kx_attn_decode_bf16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), n_q, n_kv, 128, _ptr(pos),
+                                      max_positions, _ptr(workspace), workspace.numel(), _stream()))
+
+
+def swiglu_bf16(gate, up, out):
+    _check(load().kx_swiglu_bf16(_ptr(gate), _ptr(up), _ptr(out), out.numel(), _stream()))
+
+
+def add_bf16(a, b, out):
+    _check(load().kx_add_bf16(_ptr(a), _ptr(b), _ptr(out), out.numel(), _stream()))
+
+
+def embedding_bf16(table, token, out):
+    _check(load().kx_embedding_bf16(_ptr(table), _ptr(token), _ptr(out), table.shape[0], table.shape[1], _stream()))
+
+
+def argmax_bf16(x, out_index):
+    _check(load().kx_argmax_bf16(_ptr(x), x.numel(), _ptr(out_index), _stream()))

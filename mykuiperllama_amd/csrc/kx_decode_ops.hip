@@ -1,0 +1,532 @@
+// Supporting kernels of a Qwen3-style decode step (batch 1) for gfx950: RMSNorm (optionally fused
+// with the residual add), per-head QK-norm + RoPE + KV-cache append, GQA flash-decoding (split over
+// the context, merged by log-sum-exp), SwiGLU, residual add, embedding row copy and argmax.
+// All of them are HBM- or latency-bound byte movers; arithmetic is fp32, storage bf16.
+//
+// The reference reserves layer slots for these operators (LayerRMSNorm, LayerRope, LayerMHA,
+// LayerSwiGLU, LayerAdd, LayerEmbedding: kuiper/include/op/layer.h:8-20) and names their scratch
+// buffers (model::ModelBufferType, kuiper/include/base/base.h:12-31) but implements none of them
+// except the fp32 add (kuiper/source/op/kernel/cuda/add_kernel.cu:4-12).
+#include "kx_common.h"
+
+#include <math.h>
+
+namespace kx {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+__device__ __forceinline__ void unpack8(const uint4& raw, float (&out)[8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        out[2 * i] = __uint_as_float(w[i] << 16);
+        out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+
+__device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
+    uint4 out;
+    out.x = f32_to_bf16(v[0]) | (static_cast<uint32_t>(f32_to_bf16(v[1])) << 16);
+    out.y = f32_to_bf16(v[2]) | (static_cast<uint32_t>(f32_to_bf16(v[3])) << 16);
+    out.z = f32_to_bf16(v[4]) | (static_cast<uint32_t>(f32_to_bf16(v[5])) << 16);
+    out.w = f32_to_bf16(v[6]) | (static_cast<uint32_t>(f32_to_bf16(v[7])) << 16);
+    return out;
+}
+
+// ------------------------------------------------------------------------------------------------
+// RMSNorm over rows of n elements: y = w * bf16(x * rsqrt(mean(x^2) + eps)), the rounding points of
+// the usual Qwen3 formulation (normalise in fp32, round, then scale by the bf16 gain).
+// With `delta` the row is first updated in place, x <- bf16(x + delta) (the residual add), and the
+// norm is taken of the updated row.  One workgroup per row, eight elements per thread per pass.
+// ------------------------------------------------------------------------------------------------
+constexpr int kNormThreads = 512;
+
+template <bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(uint16_t* __restrict__ x,
+                                                               const uint16_t* __restrict__ delta,
+                                                               const uint16_t* __restrict__ w,
+                                                               uint16_t* __restrict__ y, int n, float eps) {
+    __shared__ float red[kNormThreads / kWave];
+    const size_t row = blockIdx.x;
+    uint16_t* xr = x + row * n;
+    const uint16_t* dr = ADD ? delta + row * n : nullptr;
+    uint16_t* yr = y + row * n;
+    const int chunks = n >> 3;
+
+    // first pass: (update and) sum of squares; a row of up to 4096 elements stays in registers
+    float keep[8];
+    bool have = false;
+    float ss = 0.0f;
+    for (int c = threadIdx.x; c < chunks; c += kNormThreads) {
+        float v[8];
+        unpack8(reinterpret_cast<const uint4*>(xr)[c], v);
+        if (ADD) {
+            float d[8];
+            unpack8(reinterpret_cast<const uint4*>(dr)[c], d);
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = bf16_to_f32(f32_to_bf16(v[i] + d[i]));
+            reinterpret_cast<uint4*>(xr)[c] = pack8(v);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss += v[i] * v[i];
+        if (c == static_cast<int>(threadIdx.x)) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) keep[i] = v[i];
+            have = true;
+        }
+    }
+    ss = wave_sum(ss);
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / kWave; i++) total += red[i];
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(n) + eps);
+
+    for (int c = threadIdx.x; c < chunks; c += kNormThreads) {
+        float v[8], g[8];
+        if (have && c == static_cast<int>(threadIdx.x)) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = keep[i];
+        } else {
+            unpack8(reinterpret_cast<const uint4*>(xr)[c], v);
+        }
+        unpack8(reinterpret_cast<const uint4*>(w)[c], g);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = g[i] * bf16_to_f32(f32_to_bf16(v[i] * inv));
+        reinterpret_cast<uint4*>(yr)[c] = pack8(v);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-head RMSNorm (gain over head_dim = 128) of the query and key heads, rotary embedding at
+// position `pos` in the rotate-half convention, and the KV-cache append:
+//   qkv  bf16 [ (n_q + 2 n_kv) * 128 ]   = q heads | k heads | v heads, the output of a fused QKV GEMV
+//   q_out bf16 [n_q * 128]
+//   k_cache, v_cache bf16 [max_pos][n_kv][128]; row `pos` is written
+// One wave per head; lane i holds elements i and i + 64, the two partners of the rotation.
+//   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
+//   out[i + 64] = x[i+64] * cos(pos f_i) + x[i] * sin(pos f_i),     f_i = theta^(-i/64)
+// ------------------------------------------------------------------------------------------------
+constexpr int kHeadDim = 128;
+
+__global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __restrict__ qkv,
+                                                           const uint16_t* __restrict__ q_gain,
+                                                           const uint16_t* __restrict__ k_gain,
+                                                           uint16_t* __restrict__ q_out,
+                                                           uint16_t* __restrict__ k_cache,
+                                                           uint16_t* __restrict__ v_cache, int n_q, int n_kv,
+                                                           const int32_t* __restrict__ pos_ptr, float log2_theta,
+                                                           float eps) {
+    const int head = blockIdx.x * 4 + threadIdx.x / kWave;  // 0 .. n_q + 2 n_kv - 1
+    const int lane = threadIdx.x % kWave;
+    if (head >= n_q + 2 * n_kv) return;
+    const int pos = pos_ptr[0];
+    const uint16_t* src = qkv + static_cast<size_t>(head) * kHeadDim;
+    const float a = bf16_to_f32(src[lane]);
+    const float b = bf16_to_f32(src[lane + 64]);
+    if (head >= n_q + n_kv) {  // value head: straight into the cache
+        uint16_t* dst = v_cache + (static_cast<size_t>(pos) * n_kv + (head - n_q - n_kv)) * kHeadDim;
+        dst[lane] = src[lane];
+        dst[lane + 64] = src[lane + 64];
+        return;
+    }
+    const bool is_q = head < n_q;
+    const uint16_t* gain = is_q ? q_gain : k_gain;
+    const float ss = wave_sum(a * a + b * b);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(kHeadDim) + eps);
+    const float na = bf16_to_f32(gain[lane]) * bf16_to_f32(f32_to_bf16(a * inv));
+    const float nb = bf16_to_f32(gain[lane + 64]) * bf16_to_f32(f32_to_bf16(b * inv));
+    // the norm output is a bf16 tensor in the usual formulation; the rotation starts from that
+    const float xa = bf16_to_f32(f32_to_bf16(na));
+    const float xb = bf16_to_f32(f32_to_bf16(nb));
+    const float freq = exp2f(-log2_theta * static_cast<float>(lane) / 64.0f);
+    float s, c;
+    sincosf(static_cast<float>(pos) * freq, &s, &c);
+    const float oa = xa * c - xb * s;
+    const float ob = xb * c + xa * s;
+    uint16_t* dst = is_q ? q_out + static_cast<size_t>(head) * kHeadDim
+                         : k_cache + (static_cast<size_t>(pos) * n_kv + (head - n_q)) * kHeadDim;
+    dst[lane] = f32_to_bf16(oa);
+    dst[lane + 64] = f32_to_bf16(ob);
+}
+
+// ------------------------------------------------------------------------------------------------
+// GQA flash-decoding, head_dim 128, one query position.
+// Stage 1: a workgroup takes one KV head and one chunk of kAttnChunk cache positions and serves the
+// G = n_q / n_kv query heads of that KV head together, so every K and V row is read once.  Sixteen
+// lanes share a position (eight dims each, one contiguous 256-byte row per position); a wave walks
+// four positions per load.  Scores go to LDS, softmax statistics are taken per head over the chunk,
+// then V is accumulated with the chunk-local weights.  Output per (KV head, chunk): for each of the
+// G heads the unnormalised 128-vector, the chunk maximum and the chunk sum of exponentials.
+// Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
+// ------------------------------------------------------------------------------------------------
+constexpr int kAttnChunk = 128;
+constexpr int kAttnThreads = 256;
+constexpr int kMaxGroup = 8;  // query heads per KV head this kernel is instantiated for
+
+template <int G>
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, const int32_t* __restrict__ pos_ptr,
+    int nchunks, float scale) {
+    __shared__ float s_score[G][kAttnChunk];
+    __shared__ __attribute__((aligned(16))) float s_acc[kAttnThreads / kWave][G][kHeadDim];
+
+    const int kvh = blockIdx.x;
+    const int chunk = blockIdx.y;
+    const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
+    const int p0 = chunk * kAttnChunk;
+    const int tid = threadIdx.x;
+    const int sub = tid % 16;    // which eight dims of the row
+    const int slot = tid / 16;   // position slot inside the workgroup: 16 slots
+    float* out_base = part_out + (static_cast<size_t>(kvh) * nchunks + chunk) * G * kHeadDim;
+    float* ml_base = part_ml + (static_cast<size_t>(kvh) * nchunks + chunk) * G * 2;
+    if (p0 >= ctx) {
+        // a chunk past the end of the context contributes nothing: max = -inf, sum = 0
+        if (tid < G) {
+            ml_base[2 * tid] = -INFINITY;
+            ml_base[2 * tid + 1] = 0.0f;
+        }
+        return;
+    }
+
+    // the G query heads, this lane's eight dims of each
+    float qv[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        unpack8(*reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub), qv[g]);
+    }
+
+    // pass 1: scores
+    const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
+#pragma unroll
+    for (int it = 0; it < kAttnChunk / 16; it++) {
+        const int p = p0 + it * 16 + slot;
+        float kd[8];
+        if (p < ctx) {
+            unpack8(*reinterpret_cast<const uint4*>(k_cache + p * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub), kd);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) kd[i] = 0.0f;
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) d = __builtin_fmaf(qv[g][i], kd[i], d);
+            // sum over the sixteen lanes of the position
+            d += __shfl_xor(d, 8, kWave);
+            d += __shfl_xor(d, 4, kWave);
+            d += __shfl_xor(d, 2, kWave);
+            d += __shfl_xor(d, 1, kWave);
+            if (sub == 0) s_score[g][it * 16 + slot] = (p < ctx) ? d * scale : -INFINITY;
+        }
+    }
+    __syncthreads();
+
+    // softmax statistics per head over the chunk; wave w serves heads w, w + 4, ...
+    for (int g = tid / kWave; g < G; g += kAttnThreads / kWave) {
+        const int lane = tid % kWave;
+        const float s0 = s_score[g][lane];
+        const float s1 = s_score[g][lane + 64];
+        const float m = wave_max(fmaxf(s0, s1));
+        const float e0 = expf(s0 - m);
+        const float e1 = expf(s1 - m);
+        const float l = wave_sum(e0 + e1);
+        s_score[g][lane] = e0;
+        s_score[g][lane + 64] = e1;
+        if (lane == 0) {
+            ml_base[2 * g] = m;
+            ml_base[2 * g + 1] = l;
+        }
+    }
+    __syncthreads();
+
+    // pass 2: weighted sum of V rows
+    float acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
+    }
+#pragma unroll
+    for (int it = 0; it < kAttnChunk / 16; it++) {
+        const int p = p0 + it * 16 + slot;
+        if (p < ctx) {
+            float vd[8];
+            unpack8(*reinterpret_cast<const uint4*>(v_cache + p * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub), vd);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float wgt = s_score[g][it * 16 + slot];
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[g][i] = __builtin_fmaf(wgt, vd[i], acc[g][i]);
+            }
+        }
+    }
+    // the four position slots of a wave meet through lane exchanges, the four waves through LDS
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            acc[g][i] += __shfl_xor(acc[g][i], 16, kWave);
+            acc[g][i] += __shfl_xor(acc[g][i], 32, kWave);
+        }
+        if (tid % kWave < 16) {
+            float4* dst = reinterpret_cast<float4*>(&s_acc[tid / kWave][g][8 * sub]);
+            dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+            dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+        }
+    }
+    __syncthreads();
+    for (int o = tid; o < G * kHeadDim; o += kAttnThreads) {
+        const int g = o / kHeadDim;
+        const int d = o % kHeadDim;
+        float sum = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kAttnThreads / kWave; wv++) sum += s_acc[wv][g][d];
+        out_base[o] = sum;
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(kWave) void attn_decode_stage2(const float* __restrict__ part_out,
+                                                            const float* __restrict__ part_ml,
+                                                            uint16_t* __restrict__ out, int nchunks) {
+    const int head = blockIdx.x;  // query head
+    const int kvh = head / G;
+    const int g = head % G;
+    const int lane = threadIdx.x;
+    const float* ml = part_ml + static_cast<size_t>(kvh) * nchunks * G * 2;
+    float m = -INFINITY;
+    for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, ml[(static_cast<size_t>(c) * G + g) * 2]);
+    m = wave_max(m);
+    float l = 0.0f;
+    float a0 = 0.0f, a1 = 0.0f;  // dims lane and lane + 64
+    for (int c = 0; c < nchunks; c++) {
+        const float mc = ml[(static_cast<size_t>(c) * G + g) * 2];
+        const float lc = ml[(static_cast<size_t>(c) * G + g) * 2 + 1];
+        if (lc == 0.0f) continue;  // chunk past the context
+        const float f = expf(mc - m);
+        l += lc * f;
+        const float* po = part_out + ((static_cast<size_t>(kvh) * nchunks + c) * G + g) * kHeadDim;
+        a0 += po[lane] * f;
+        a1 += po[lane + 64] * f;
+    }
+    const float inv = 1.0f / l;
+    out[static_cast<size_t>(head) * kHeadDim + lane] = f32_to_bf16(a0 * inv);
+    out[static_cast<size_t>(head) * kHeadDim + lane + 64] = f32_to_bf16(a1 * inv);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Elementwise: SwiGLU, residual add.  Eight elements per thread, grid-stride.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ gate,
+                                                     const uint16_t* __restrict__ up,
+                                                     uint16_t* __restrict__ out, int chunks) {
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += gridDim.x * blockDim.x) {
+        float g[8], u[8];
+        unpack8(reinterpret_cast<const uint4*>(gate)[c], g);
+        unpack8(reinterpret_cast<const uint4*>(up)[c], u);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // silu(g) is a bf16 tensor before it meets `up` in the usual formulation
+            const float act = bf16_to_f32(f32_to_bf16(g[i] / (1.0f + expf(-g[i]))));
+            g[i] = act * u[i];
+        }
+        reinterpret_cast<uint4*>(out)[c] = pack8(g);
+    }
+}
+
+__global__ __launch_bounds__(256) void add_bf16_kernel(const uint16_t* __restrict__ a,
+                                                       const uint16_t* __restrict__ b,
+                                                       uint16_t* __restrict__ out, int chunks) {
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += gridDim.x * blockDim.x) {
+        float x[8], y[8];
+        unpack8(reinterpret_cast<const uint4*>(a)[c], x);
+        unpack8(reinterpret_cast<const uint4*>(b)[c], y);
+#pragma unroll
+        for (int i = 0; i < 8; i++) x[i] += y[i];
+        reinterpret_cast<uint4*>(out)[c] = pack8(x);
+    }
+}
+
+__global__ __launch_bounds__(256) void embedding_kernel(const uint16_t* __restrict__ table,
+                                                        const int32_t* __restrict__ token_ptr,
+                                                        uint16_t* __restrict__ out, int chunks, int vocab) {
+    int token = token_ptr[0];
+    token = token < 0 ? 0 : (token >= vocab ? vocab - 1 : token);
+    const uint4* row = reinterpret_cast<const uint4*>(table + static_cast<size_t>(token) * chunks * 8);
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += gridDim.x * blockDim.x) {
+        reinterpret_cast<uint4*>(out)[c] = row[c];
+    }
+}
+
+// argmax over n bf16 values, first index on ties, NaN ignored; one workgroup.
+constexpr int kArgmaxThreads = 1024;
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* __restrict__ x, int n,
+                                                               int32_t* __restrict__ out) {
+    __shared__ float s_val[kArgmaxThreads / kWave];
+    __shared__ int s_idx[kArgmaxThreads / kWave];
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += kArgmaxThreads) {
+        const float v = bf16_to_f32(x[i]);
+        if (v > best) {  // ascending i per thread: the first maximum wins; NaN never compares greater
+            best = v;
+            best_i = i;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, kWave);
+        const int oi = __shfl_xor(best_i, off, kWave);
+        if (ov > best || (ov == best && oi < best_i)) {
+            best = ov;
+            best_i = oi;
+        }
+    }
+    if (threadIdx.x % kWave == 0) {
+        s_val[threadIdx.x / kWave] = best;
+        s_idx[threadIdx.x / kWave] = best_i;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kArgmaxThreads / kWave; w++) {
+            if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
+                best = s_val[w];
+                best_i = s_idx[w];
+            }
+        }
+        out[0] = best_i == 0x7fffffff ? 0 : best_i;
+    }
+}
+
+inline bool aligned16(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) % 16) == 0;
+}
+
+}  // namespace
+}  // namespace kx
+
+extern "C" int kx_rmsnorm_bf16(const uint16_t* x, const uint16_t* gain, uint16_t* y, int32_t rows, int32_t n,
+                               float eps, void* stream) {
+    if (!x || !gain || !y) return KX_ERR_NULL_POINTER;
+    if (rows < 1 || n < 8 || (n % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(x) || !kx::aligned16(gain) || !kx::aligned16(y)) return KX_ERR_ALIGNMENT;
+    hipLaunchKernelGGL((kx::rmsnorm_kernel<false>), dim3(rows), dim3(kx::kNormThreads), 0, kx::as_stream(stream),
+                       const_cast<uint16_t*>(x), static_cast<const uint16_t*>(nullptr), gain, y, n, eps);
+    return kx::launch_status();
+}
+
+extern "C" int kx_add_rmsnorm_bf16(uint16_t* x_inout, const uint16_t* delta, const uint16_t* gain, uint16_t* y,
+                                   int32_t rows, int32_t n, float eps, void* stream) {
+    if (!x_inout || !delta || !gain || !y) return KX_ERR_NULL_POINTER;
+    if (rows < 1 || n < 8 || (n % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(x_inout) || !kx::aligned16(delta) || !kx::aligned16(gain) || !kx::aligned16(y)) {
+        return KX_ERR_ALIGNMENT;
+    }
+    hipLaunchKernelGGL((kx::rmsnorm_kernel<true>), dim3(rows), dim3(kx::kNormThreads), 0, kx::as_stream(stream),
+                       x_inout, delta, gain, y, n, eps);
+    return kx::launch_status();
+}
+
+extern "C" int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain,
+                                    uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int32_t n_q_heads,
+                                    int32_t n_kv_heads, int32_t head_dim, const int32_t* pos, float rope_theta,
+                                    float eps, void* stream) {
+    if (!qkv || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) return KX_ERR_NULL_POINTER;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || !(rope_theta > 1.0f)) return KX_ERR_BAD_SHAPE;
+    const int heads = n_q_heads + 2 * n_kv_heads;
+    hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4), dim3(256), 0, kx::as_stream(stream), qkv,
+                       q_gain, k_gain, q_out, k_cache, v_cache, n_q_heads, n_kv_heads, pos, log2f(rope_theta), eps);
+    return kx::launch_status();
+}
+
+extern "C" size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head_dim, int32_t max_positions) {
+    if (n_q_heads < 1 || head_dim != kx::kHeadDim || max_positions < 1) return 0;
+    const size_t nchunks = (static_cast<size_t>(max_positions) + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    return nchunks * n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
+}
+
+extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                                   uint16_t* out, int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim,
+                                   const int32_t* pos, int32_t max_positions, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+    if (!q || !k_cache || !v_cache || !out || !pos || !workspace) return KX_ERR_NULL_POINTER;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || (n_q_heads % n_kv_heads) != 0 ||
+        max_positions < 1) {
+        return KX_ERR_BAD_SHAPE;
+    }
+    const int G = n_q_heads / n_kv_heads;
+    if (G != 1 && G != 2 && G != 4 && G != 8) return KX_ERR_BAD_SHAPE;
+    if (workspace_bytes < kx_attn_decode_workspace_bytes(n_q_heads, head_dim, max_positions)) return KX_ERR_WORKSPACE;
+    if (!kx::aligned16(q) || !kx::aligned16(k_cache) || !kx::aligned16(v_cache) || !kx::aligned16(workspace)) {
+        return KX_ERR_ALIGNMENT;
+    }
+    const int nchunks = (max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    float* part_out = static_cast<float*>(workspace);
+    float* part_ml = part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
+    const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
+    hipStream_t s = kx::as_stream(stream);
+    dim3 grid1(n_kv_heads, nchunks);
+#define KX_ATTN(GG)                                                                                           \
+    hipLaunchKernelGGL((kx::attn_decode_stage1<GG>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache, v_cache, \
+                       part_out, part_ml, n_kv_heads, pos, nchunks, scale);                                    \
+    hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kWave), 0, s, part_out, part_ml,  \
+                       out, nchunks)
+    if (G == 1) { KX_ATTN(1); } else if (G == 2) { KX_ATTN(2); } else if (G == 4) { KX_ATTN(4); } else { KX_ATTN(8); }
+#undef KX_ATTN
+    return kx::launch_status();
+}
+
+extern "C" int kx_swiglu_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int32_t n, void* stream) {
+    if (!gate || !up || !out) return KX_ERR_NULL_POINTER;
+    if (n < 8 || (n % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(gate) || !kx::aligned16(up) || !kx::aligned16(out)) return KX_ERR_ALIGNMENT;
+    const int chunks = n / 8;
+    int blocks = (chunks + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(kx::swiglu_kernel, dim3(blocks), dim3(256), 0, kx::as_stream(stream), gate, up, out, chunks);
+    return kx::launch_status();
+}
+
+extern "C" int kx_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int32_t n, void* stream) {
+    if (!a || !b || !out) return KX_ERR_NULL_POINTER;
+    if (n < 8 || (n % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(a) || !kx::aligned16(b) || !kx::aligned16(out)) return KX_ERR_ALIGNMENT;
+    const int chunks = n / 8;
+    int blocks = (chunks + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(kx::add_bf16_kernel, dim3(blocks), dim3(256), 0, kx::as_stream(stream), a, b, out, chunks);
+    return kx::launch_status();
+}
+
+extern "C" int kx_embedding_bf16(const uint16_t* table, const int32_t* token, uint16_t* out, int32_t vocab,
+                                 int32_t dim, void* stream) {
+    if (!table || !token || !out) return KX_ERR_NULL_POINTER;
+    if (vocab < 1 || dim < 8 || (dim % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(table) || !kx::aligned16(out)) return KX_ERR_ALIGNMENT;
+    const int chunks = dim / 8;
+    hipLaunchKernelGGL(kx::embedding_kernel, dim3((chunks + 255) / 256), dim3(256), 0, kx::as_stream(stream), table,
+                       token, out, chunks, vocab);
+    return kx::launch_status();
+}
+
+extern "C" int kx_argmax_bf16(const uint16_t* x, int32_t n, int32_t* out_index, void* stream) {
+    if (!x || !out_index) return KX_ERR_NULL_POINTER;
+    if (n < 1) return KX_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(kx::argmax_kernel, dim3(1), dim3(kx::kArgmaxThreads), 0, kx::as_stream(stream), x, n, out_index);
+    return kx::launch_status();
+}

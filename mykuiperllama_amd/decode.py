@@ -1,0 +1,172 @@
+"""Qwen3-shaped decode step (batch 1) assembled from the C ABI entry points.
+
+Plumbing for the benchmark and for the end-to-end parity test: random-init (or caller-supplied)
+INT4 AWQ weights, bf16 KV cache, and the launch sequence of one token.  The reference has no model
+code (its model/ directory is absent), so this is not a port of anything; the operator order is
+the usual pre-norm decoder with per-head QK-norm:
+
+  x = embed[token]
+  per layer:  h = rmsnorm(x);  qkv = Wqkv h;  q,k <- head-norm + rope, k,v -> cache;  a = attn(q);
+              x += Wo a;  h = rmsnorm(x);  x += Wdown( silu(Wgate h) * (Wup h) )
+  logits = lm_head rmsnorm(x);  next = argmax(logits)
+
+q/k/v share one fused GEMV (N = (n_q + 2 n_kv) * 128) and gate/up another (N = 2 * intermediate): the
+packed tensors of the separate projections are concatenated along N when the weights are loaded
+(rows are laid end to end; the nibble order inside a word is untouched).  The residual add is fused
+into the next RMSNorm.  Every launch goes to torch's current stream, so a step can be captured in
+a HIP graph; token and position live in device memory for that reason.
+"""
+from dataclasses import dataclass
+
+from . import capi
+
+
+@dataclass
+class ModelConfig:
+    layers: int
+    hidden: int
+    intermediate: int
+    n_q: int
+    n_kv: int
+    vocab: int
+    head_dim: int = 128
+    rope_theta: float = 1e6
+    eps: float = 1e-6
+    group: int = 128
+
+    @property
+    def qkv_out(self):
+        return (self.n_q + 2 * self.n_kv) * self.head_dim
+
+
+QWEN3_8B = ModelConfig(layers=36, hidden=4096, intermediate=12288, n_q=32, n_kv=8, vocab=151936)
+QWEN3_32B = ModelConfig(layers=64, hidden=5120, intermediate=25600, n_q=64, n_kv=8, vocab=151936)
+
+
+def _rand_awq(torch, K, N, group, gen):
+    qw = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+    qz = torch.randint(-2**31, 2**31 - 1, (K // group, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+    # scales sized so that activations keep O(1) magnitude through the layers: |w| ~ 4.6 s, fan-in K
+    s = (torch.rand((K // group, N), device="cuda", generator=gen) * 0.5 + 0.75) * (1.0 / (4.6 * K ** 0.5))
+    return qw, s.half(), qz
+
+
+class DecodeModel:
+    """Weights, caches and scratch buffers of one model on the GPU."""
+
+    def __init__(self, cfg, max_positions, weights=None, seed=20251125):
+        import torch
+        self.torch = torch
+        self.cfg = cfg
+        self.max_positions = max_positions
+        c = cfg
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        bf = torch.bfloat16
+
+        def rand_bf16(shape, std):
+            return (torch.randn(shape, device="cuda", generator=gen) * std).to(bf)
+
+        if weights is None:
+            self.layers = []
+            for _ in range(c.layers):
+                self.layers.append({
+                    "qkv": _rand_awq(torch, c.hidden, c.qkv_out, c.group, gen),
+                    "o": _rand_awq(torch, c.n_q * c.head_dim, c.hidden, c.group, gen),
+                    "gateup": _rand_awq(torch, c.hidden, 2 * c.intermediate, c.group, gen),
+                    "down": _rand_awq(torch, c.intermediate, c.hidden, c.group, gen),
+                    "in_norm": 1 + rand_bf16((c.hidden,), 0.02),
+                    "post_norm": 1 + rand_bf16((c.hidden,), 0.02),
+                    "q_norm": 1 + rand_bf16((c.head_dim,), 0.02),
+                    "k_norm": 1 + rand_bf16((c.head_dim,), 0.02),
+                })
+            self.embed = rand_bf16((c.vocab, c.hidden), 1.0)
+            self.lm_head = rand_bf16((c.vocab, c.hidden), 0.02)
+            self.final_norm = 1 + rand_bf16((c.hidden,), 0.02)
+        else:
+            self.layers = weights["layers"]
+            self.embed = weights["embed"]
+            self.lm_head = weights["lm_head"]
+            self.final_norm = weights["final_norm"]
+
+        self.k_cache = [torch.zeros((max_positions, c.n_kv, c.head_dim), dtype=bf, device="cuda") for _ in range(c.layers)]
+        self.v_cache = [torch.zeros((max_positions, c.n_kv, c.head_dim), dtype=bf, device="cuda") for _ in range(c.layers)]
+
+        def buf(n):
+            return torch.zeros((1, n), dtype=bf, device="cuda")
+
+        self.x = buf(c.hidden)
+        self.h = buf(c.hidden)
+        self.qkv = buf(c.qkv_out)
+        self.q = buf(c.n_q * c.head_dim)
+        self.attn = buf(c.n_q * c.head_dim)
+        self.o = buf(c.hidden)
+        self.gu = buf(2 * c.intermediate)
+        self.act = buf(c.intermediate)
+        self.down = buf(c.hidden)
+        self.logits = buf(c.vocab)
+        self.token = torch.zeros(1, dtype=torch.int32, device="cuda")
+        self.pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+        self.next_token = torch.zeros(1, dtype=torch.int32, device="cuda")
+        big_k = max(c.hidden, c.intermediate, c.n_q * c.head_dim)
+        big_n = max(c.qkv_out, 2 * c.intermediate, c.hidden)
+        self.gemv_ws = capi.make_workspace(1, big_k, big_n)
+        self.attn_ws = capi.attn_decode_workspace(c.n_q, max_positions)
+
+    def prefill_cache_random(self, ctx, seed=7):
+        """Fill cache rows 0 .. ctx-1 with N(0,1), as the benchmark configurations ask."""
+        torch = self.torch
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        for kc, vc in zip(self.k_cache, self.v_cache):
+            kc[:ctx] = torch.randn(kc[:ctx].shape, device="cuda", generator=gen).to(torch.bfloat16)
+            vc[:ctx] = torch.randn(vc[:ctx].shape, device="cuda", generator=gen).to(torch.bfloat16)
+
+    def set_input(self, token, pos):
+        self.token.fill_(token)
+        self.pos.fill_(pos)
+
+    def _awq(self, x, w, y):
+        capi.gemv_awq_bf16(x, w[0], w[1], w[2], y, self.cfg.group, self.gemv_ws)
+
+    def step(self, with_lm_head=True):
+        """Enqueue one decode step on torch's current stream (no synchronisation)."""
+        c = self.cfg
+        capi.embedding_bf16(self.embed, self.token, self.x)
+        for li, L in enumerate(self.layers):
+            if li == 0:
+                capi.rmsnorm_bf16(self.x, L["in_norm"], self.h, c.eps)
+            else:
+                capi.add_rmsnorm_bf16(self.x, self.down, L["in_norm"], self.h, c.eps)
+            self._awq(self.h, L["qkv"], self.qkv)
+            capi.qk_norm_rope_bf16(self.qkv, L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
+                                   c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps)
+            capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
+                                  self.max_positions, self.attn_ws)
+            self._awq(self.attn, L["o"], self.o)
+            capi.add_rmsnorm_bf16(self.x, self.o, L["post_norm"], self.h, c.eps)
+            self._awq(self.h, L["gateup"], self.gu)
+            capi.swiglu_bf16(self.gu[:, : c.intermediate], self.gu[:, c.intermediate:], self.act)
+            self._awq(self.act, L["down"], self.down)
+        capi.add_rmsnorm_bf16(self.x, self.down, self.final_norm, self.h, c.eps)
+        if with_lm_head:
+            capi.gemv_bf16(self.h, self.lm_head, self.logits)
+            capi.argmax_bf16(self.logits, self.next_token)
+
+    def launches_per_step(self, with_lm_head=True):
+        return 1 + self.cfg.layers * 10 + 1 + (2 if with_lm_head else 0)
+
+
+def step_bytes(cfg, ctx, with_lm_head=True):
+    """Algorithmic HBM bytes of one decode step: packed projections + KV read (+ bf16 lm_head)."""
+    from .synth import awq_gemv_bytes
+    per_layer = (awq_gemv_bytes(1, cfg.hidden, cfg.n_q * cfg.head_dim, cfg.group)
+                 + 2 * awq_gemv_bytes(1, cfg.hidden, cfg.n_kv * cfg.head_dim, cfg.group)
+                 + awq_gemv_bytes(1, cfg.n_q * cfg.head_dim, cfg.hidden, cfg.group)
+                 + 2 * awq_gemv_bytes(1, cfg.hidden, cfg.intermediate, cfg.group)
+                 + awq_gemv_bytes(1, cfg.intermediate, cfg.hidden, cfg.group))
+    kv = 2 * ctx * cfg.n_kv * cfg.head_dim * 2
+    total = cfg.layers * (per_layer + kv)
+    if with_lm_head:
+        total += cfg.vocab * cfg.hidden * 2
+    return total

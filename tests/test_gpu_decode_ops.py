@@ -1,0 +1,185 @@
+"""GPU parity of the decode-step supporting kernels against fp32 torch references on the CPU.
+
+These are floating-point kernels with bf16 storage, so the reference is the closed form evaluated
+in fp32 by torch and rounded where the kernel rounds; tolerances are stated per test.  The
+conventions that a closed form cannot pin by itself (rotate-half pairing, norm before rotation,
+rounding points of RMSNorm) are checked against the Qwen3 modelling code that ships with the
+installed transformers package (a library oracle; nothing is downloaded).
+"""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch as _t
+    assert _t.cuda.is_available()
+    _t.manual_seed(1234)
+    return _t
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from mykuiperllama_amd import capi as _c
+    _c.load()
+    return _c
+
+
+def ulp_diff(torch, a, b):
+    """Distance in bf16 units-in-the-last-place between two bf16 tensors (same sign region)."""
+    ia = a.view(torch.int16).to(torch.int32)
+    ib = b.view(torch.int16).to(torch.int32)
+    return (ia - ib).abs()
+
+
+def ref_rmsnorm(torch, x, gain, eps):
+    xf = x.float()
+    normed = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)
+    return gain * normed  # bf16 * bf16 -> bf16, the rounding points of Qwen3RMSNorm
+
+
+@pytest.mark.parametrize("rows,n", [(1, 4096), (1, 5120), (3, 1024), (2, 128), (1, 8)])
+def test_rmsnorm_matches_reference_and_transformers(capi, torch, rows, n):
+    eps = 1e-6
+    x = (torch.randn(rows, n) * 3).bfloat16()
+    gain = (1 + 0.1 * torch.randn(n)).bfloat16()
+    y = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    capi.rmsnorm_bf16(x.cuda(), gain.cuda(), y, eps)
+    torch.cuda.synchronize()
+    ref = ref_rmsnorm(torch, x, gain, eps)
+    d = ulp_diff(torch, y.cpu(), ref)
+    assert d.max() <= 1 and (d == 0).float().mean() > 0.99  # rsqrt vs 1/sqrt may flip a rounding
+    from transformers.models.qwen3.modeling_qwen3 import Qwen3RMSNorm
+    mod = Qwen3RMSNorm(n, eps=eps).to(torch.bfloat16)
+    with torch.no_grad():
+        mod.weight.copy_(gain)
+        hf = mod(x)
+    assert ulp_diff(torch, y.cpu(), hf).max() <= 1
+
+
+def test_add_rmsnorm_updates_the_residual_in_place(capi, torch):
+    n, eps = 4096, 1e-6
+    x = torch.randn(1, n).bfloat16()
+    delta = torch.randn(1, n).bfloat16()
+    gain = (1 + 0.1 * torch.randn(n)).bfloat16()
+    xd = x.cuda().clone()
+    y = torch.empty(1, n, dtype=torch.bfloat16, device="cuda")
+    capi.add_rmsnorm_bf16(xd, delta.cuda(), gain.cuda(), y, eps)
+    torch.cuda.synchronize()
+    x_new = x + delta  # bf16 addition rounds once, like the kernel
+    assert torch.equal(xd.cpu(), x_new)
+    assert ulp_diff(torch, y.cpu(), ref_rmsnorm(torch, x_new, gain, eps)).max() <= 1
+
+
+@pytest.mark.parametrize("n_q,n_kv,pos", [(32, 8, 0), (32, 8, 4096), (64, 8, 8191), (4, 2, 17), (2, 2, 1)])
+def test_qk_norm_rope_and_cache_append(capi, torch, n_q, n_kv, pos):
+    theta, eps, D = 1e6, 1e-6, 128
+    max_pos = pos + 3
+    qkv = torch.randn((n_q + 2 * n_kv) * D).bfloat16()
+    qg = (1 + 0.1 * torch.randn(D)).bfloat16()
+    kg = (1 + 0.1 * torch.randn(D)).bfloat16()
+    q_out = torch.zeros(n_q, D, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(max_pos, n_kv, D, dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros(max_pos, n_kv, D, dtype=torch.bfloat16, device="cuda")
+    pos_t = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    capi.qk_norm_rope_bf16(qkv.cuda(), qg.cuda(), kg.cuda(), q_out, kc, vc, n_q, n_kv, pos_t, theta, eps)
+    torch.cuda.synchronize()
+
+    q = qkv[: n_q * D].view(n_q, D)
+    k = qkv[n_q * D:(n_q + n_kv) * D].view(n_kv, D)
+    v = qkv[(n_q + n_kv) * D:].view(n_kv, D)
+    qn = ref_rmsnorm(torch, q, qg, eps).float()
+    kn = ref_rmsnorm(torch, k, kg, eps).float()
+    inv_freq = 1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = pos * inv_freq
+    cos = torch.cat([ang, ang]).cos()
+    sin = torch.cat([ang, ang]).sin()
+
+    def rot(t):
+        return torch.cat([-t[..., D // 2:], t[..., : D // 2]], dim=-1)
+
+    q_ref = qn * cos + rot(qn) * sin
+    k_ref = kn * cos + rot(kn) * sin
+    # fp32 reference, one bf16 rounding at the end: within one ulp of the output scale
+    scale_q = q_ref.abs().max().item()
+    assert (q_out.cpu().float() - q_ref).abs().max() <= 2.0 ** (math.floor(math.log2(scale_q)) - 7)
+    assert (kc[pos].cpu().float() - k_ref).abs().max() <= 2.0 ** (math.floor(math.log2(k_ref.abs().max().item())) - 7)
+    assert torch.equal(vc[pos].cpu(), v)
+    other = [p for p in range(max_pos) if p != pos]
+    assert not kc[other].any() and not vc[other].any()  # only row `pos` is written
+
+    # convention check against the library: bf16 cos/sin there, so a looser bound
+    from transformers.models.qwen3.modeling_qwen3 import apply_rotary_pos_emb
+    qh, kh = apply_rotary_pos_emb(qn.bfloat16()[None, :, None, :], kn.bfloat16()[None, :, None, :],
+                                  cos.bfloat16()[None, None, :], sin.bfloat16()[None, None, :])
+    assert (q_out.cpu().float() - qh[0, :, 0].float()).abs().max() <= 0.03 * max(scale_q, 1.0)
+    assert (kc[pos].cpu().float() - kh[0, :, 0].float()).abs().max() <= 0.03 * max(k_ref.abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (8, 4), (4, 4)])
+@pytest.mark.parametrize("ctx", [1, 5, 128, 129, 1000, 4097])
+def test_attention_decode_matches_fp32_softmax(capi, torch, n_q, n_kv, ctx):
+    D = 128
+    max_pos = 4224
+    G = n_q // n_kv
+    q = torch.randn(n_q, D).bfloat16()
+    kc = torch.randn(max_pos, n_kv, D).bfloat16()
+    vc = torch.randn(max_pos, n_kv, D).bfloat16()
+    out = torch.full((n_q, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    pos_t = torch.tensor([ctx - 1], dtype=torch.int32, device="cuda")
+    ws = capi.attn_decode_workspace(n_q, max_pos)
+    capi.attn_decode_bf16(q.cuda(), kc.cuda(), vc.cuda(), out, n_q, n_kv, pos_t, max_pos, ws)
+    torch.cuda.synchronize()
+    kf = kc[:ctx].float().repeat_interleave(G, dim=1)  # [ctx, n_q, D]
+    vf = vc[:ctx].float().repeat_interleave(G, dim=1)
+    scores = torch.einsum("hd,phd->hp", q.float(), kf) / math.sqrt(D)
+    ref = torch.einsum("hp,phd->hd", torch.softmax(scores, dim=-1), vf)
+    got = out.cpu().float()
+    assert torch.isfinite(got).all()
+    err = (got - ref).norm() / ref.norm()
+    assert err <= 3e-3  # the bf16 store alone is ~1.6e-3
+    assert (got - ref).abs().max() <= 2 * 2.0 ** (math.floor(math.log2(ref.abs().max().item())) - 7)
+
+
+def test_swiglu_add_embedding_argmax(capi, torch):
+    n = 12288
+    g = (torch.randn(n) * 2).bfloat16()
+    u = torch.randn(n).bfloat16()
+    out = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    capi.swiglu_bf16(g.cuda(), u.cuda(), out)
+    torch.cuda.synchronize()
+    ref = torch.nn.functional.silu(g.float()).bfloat16() * u
+    d = ulp_diff(torch, out.cpu(), ref)
+    assert d.max() <= 1 and (d == 0).float().mean() > 0.98  # expf vs torch's exp may flip a rounding
+
+    a = torch.randn(4096).bfloat16()
+    b = torch.randn(4096).bfloat16()
+    capi.add_bf16(a.cuda(), b.cuda(), out[:4096])
+    torch.cuda.synchronize()
+    assert torch.equal(out[:4096].cpu(), a + b)
+
+    table = torch.randn(1000, 512).bfloat16().cuda()
+    row = torch.empty(512, dtype=torch.bfloat16, device="cuda")
+    for tok in (0, 7, 999, 5000, -3):  # out-of-range tokens clamp
+        capi.embedding_bf16(table, torch.tensor([tok], dtype=torch.int32, device="cuda"), row)
+        torch.cuda.synchronize()
+        assert torch.equal(row, table[min(max(tok, 0), 999)])
+
+    logits = torch.randn(151936).bfloat16()
+    logits[77777] = 50.0
+    idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    capi.argmax_bf16(logits.cuda(), idx)
+    torch.cuda.synchronize()
+    assert idx.item() == 77777
+    logits[123] = 50.0  # a tie: the first index wins
+    capi.argmax_bf16(logits.cuda(), idx)
+    torch.cuda.synchronize()
+    assert idx.item() == 123
+    logits[5] = float("nan")  # NaN is ignored
+    capi.argmax_bf16(logits.cuda(), idx)
+    torch.cuda.synchronize()
+    assert idx.item() == 123
