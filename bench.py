@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-passes", type=int, default=30)
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the Qwen3-8B decode-step measurement")
+    ap.add_argument("--decode-32b", action="store_true", help="also run the Qwen3-32B-shaped decode step")
+    ap.add_argument("--decode-steps", type=int, default=60)
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection workload: one 256 MiB device copy (known traffic, for scaling the "
                          "counters) followed by a few cold launches per projection shape; prints no metric")
@@ -63,6 +66,7 @@ class WeightSet:
 
 def timed_region(torch, launch_steps, steps, warmup, eager, steps_per_graph):
     """Run `warmup` untimed steps, then exactly `steps` timed ones; returns seconds (events)."""
+    torch.cuda.synchronize()  # tensors were initialised on the default stream; the launches below use another
     stream = torch.cuda.current_stream()
     if eager:
         launch_steps(0, warmup)
@@ -122,6 +126,34 @@ def cpu_baseline(passes):
             "sample": f"{passes} passes over the seven Qwen3-8B projections at M=1 (seeded inputs), "
                       f"oracle/kx_oracle.c kxo_gemv_awq_f32, gcc -O3 -march=x86-64-v3, one thread, "
                       f"host has {os.cpu_count()} logical cpus"}
+
+
+def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager):
+    """Tokens/s of a full random-init decode step (batch 1, KV cache pre-filled at `ctx`)."""
+    from mykuiperllama_amd import decode
+    cfg = {"qwen3-8b": decode.QWEN3_8B, "qwen3-32b": decode.QWEN3_32B}[cfg_name]
+    model = decode.DecodeModel(cfg, max_positions=ctx + 128)
+    model.prefill_cache_random(ctx)
+    model.set_input(1, ctx)  # every timed step decodes position `ctx` against ctx cached positions
+    out = {"model": cfg_name, "context": ctx, "steps": steps, "launch": "eager" if eager else "hipGraph replay",
+           "weights": "random-init INT4 AWQ group 128 (q/k/v and gate/up fused along N), bf16 embedding and lm_head"}
+    for with_head in (True, False):
+        def launch(first, count, with_head=with_head):
+            for _ in range(count):
+                model.step(with_lm_head=with_head)
+        sec = timed_region(torch, launch, steps, warmup, eager, 4)
+        key = "with_lm_head" if with_head else "without_lm_head"
+        nbytes = decode.step_bytes(cfg, ctx, with_head)
+        out[key] = {"tokens_per_s": round(steps / sec, 1), "ms_per_token": round(sec / steps * 1e3, 4),
+                    "algorithmic_GB_per_token": round(nbytes / 1e9, 3),
+                    "GB/s": round(nbytes / (sec / steps) / 1e9, 1),
+                    "pct_of_8TBps": round(nbytes / (sec / steps) / 1e9 / HBM_PEAK_GBPS * 100, 2),
+                    "launches_per_token": model.launches_per_step(with_head)}
+    torch.cuda.synchronize()
+    out["next_token_finite"] = bool(torch.isfinite(model.logits.float()).all().item())
+    del model
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -219,6 +251,15 @@ def main():
     }
     if per_shape is not None:
         out["per_shape"] = per_shape
+    if not args.no_decode:
+        del sets
+        torch.cuda.empty_cache()
+        d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager)
+        out["decode_tok_s"] = d8["with_lm_head"]["tokens_per_s"]
+        out["decode"] = {"qwen3-8b ctx4096": d8}
+        if args.decode_32b:
+            out["decode"]["qwen3-32b ctx8192"] = decode_benchmark(torch, "qwen3-32b", 8192, args.decode_steps, 8,
+                                                                  args.eager)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_passes)
     print(json.dumps(out))
