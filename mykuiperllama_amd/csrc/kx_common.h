@@ -45,6 +45,49 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return static_cast<float>(v);
 }
 
+// Lane exchanges inside a row of 16 lanes ride on the VALU's data-parallel-primitive operand path
+// (one instruction for move + add), where a ds_bpermute costs an LDS round trip of ~100 cycles that a
+// dependent chain cannot hide.  CTRL 0x120 + n rotates a row right by n lanes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// every lane of a 16-lane row receives the row's sum (lanes may differ in the last bit: each adds
+// the same sixteen numbers in its own rotated order)
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0x128>(v);
+    v += dpp_move<0x124>(v);
+    v += dpp_move<0x122>(v);
+    v += dpp_move<0x121>(v);
+    return v;
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0x128>(v));
+    v = fmaxf(v, dpp_move<0x124>(v));
+    v = fmaxf(v, dpp_move<0x122>(v));
+    v = fmaxf(v, dpp_move<0x121>(v));
+    return v;
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// wave-wide reductions, the same value in every lane: rows by rotation, the four rows through
+// scalar registers
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
+}
+
 inline hipStream_t as_stream(void* s) {
     return static_cast<hipStream_t>(s);
 }

@@ -14,18 +14,6 @@
 namespace kx {
 namespace {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
-}
-
 __device__ __forceinline__ void unpack8(const uint4& raw, float (&out)[8]) {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -172,25 +160,56 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 // G heads the unnormalised 128-vector, the chunk maximum and the chunk sum of exponentials.
 // Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
 // ------------------------------------------------------------------------------------------------
-constexpr int kAttnChunk = 128;
+constexpr int kAttnChunk = 64;
 constexpr int kAttnThreads = 256;
+constexpr int kAttnSlots = kAttnThreads / 16;  // cache positions a workgroup handles side by side
+constexpr int kAccHeads = 4;                   // heads whose slot sums fit in LDS together (32 KiB)
 constexpr int kMaxGroup = 8;  // query heads per KV head this kernel is instantiated for
 
 template <int G>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, const int32_t* __restrict__ pos_ptr,
-    int nchunks, float scale) {
+    int nchunks, int max_positions, float scale) {
     __shared__ float s_score[G][kAttnChunk];
-    __shared__ __attribute__((aligned(16))) float s_acc[kAttnThreads / kWave][G][kHeadDim];
+    __shared__ __attribute__((aligned(16))) float s_acc[kAttnSlots][G < kAccHeads ? G : kAccHeads][kHeadDim];
 
-    const int kvh = blockIdx.x;
-    const int chunk = blockIdx.y;
-    const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
+    const int kvh = blockIdx.y;
+    const int chunk = blockIdx.x;
     const int p0 = chunk * kAttnChunk;
     const int tid = threadIdx.x;
     const int sub = tid % 16;    // which eight dims of the row
     const int slot = tid / 16;   // position slot inside the workgroup: 16 slots
+
+    // Every K and V row of this lane is requested before anything is consumed, and the addresses do
+    // not depend on *pos: any row below max_positions exists, rows past the context are masked once
+    // the position has arrived.  The chunk then costs one memory round trip.
+    const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
+    constexpr int ITERS = kAttnChunk / 16;
+    u32x4 kraw[ITERS], vraw[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int p = p0 + it * 16 + slot;
+        const int pc = p < max_positions ? p : max_positions - 1;
+        kraw[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+            k_cache + pc * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub));
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int p = p0 + it * 16 + slot;
+        const int pc = p < max_positions ? p : max_positions - 1;
+        vraw[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+            v_cache + pc * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub));
+    }
+    // the G query heads, this lane's eight dims of each
+    float qv[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        unpack8(*reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub), qv[g]);
+    }
+    const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
+    __builtin_amdgcn_sched_barrier(0);
+
     float* out_base = part_out + (static_cast<size_t>(kvh) * nchunks + chunk) * G * kHeadDim;
     float* ml_base = part_ml + (static_cast<size_t>(kvh) * nchunks + chunk) * G * 2;
     if (p0 >= ctx) {
@@ -202,35 +221,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         return;
     }
 
-    // the G query heads, this lane's eight dims of each
-    float qv[G][8];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        unpack8(*reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub), qv[g]);
-    }
-
     // pass 1: scores
-    const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
 #pragma unroll
-    for (int it = 0; it < kAttnChunk / 16; it++) {
+    for (int it = 0; it < ITERS; it++) {
         const int p = p0 + it * 16 + slot;
         float kd[8];
-        if (p < ctx) {
-            unpack8(*reinterpret_cast<const uint4*>(k_cache + p * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub), kd);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) kd[i] = 0.0f;
-        }
+        unpack8(make_uint4(kraw[it].x, kraw[it].y, kraw[it].z, kraw[it].w), kd);
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float d = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) d = __builtin_fmaf(qv[g][i], kd[i], d);
-            // sum over the sixteen lanes of the position
-            d += __shfl_xor(d, 8, kWave);
-            d += __shfl_xor(d, 4, kWave);
-            d += __shfl_xor(d, 2, kWave);
-            d += __shfl_xor(d, 1, kWave);
+            d = row16_sum(d);  // the sixteen lanes of the position
             if (sub == 0) s_score[g][it * 16 + slot] = (p < ctx) ? d * scale : -INFINITY;
         }
     }
@@ -239,14 +241,23 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // softmax statistics per head over the chunk; wave w serves heads w, w + 4, ...
     for (int g = tid / kWave; g < G; g += kAttnThreads / kWave) {
         const int lane = tid % kWave;
-        const float s0 = s_score[g][lane];
-        const float s1 = s_score[g][lane + 64];
-        const float m = wave_max(fmaxf(s0, s1));
-        const float e0 = expf(s0 - m);
-        const float e1 = expf(s1 - m);
-        const float l = wave_sum(e0 + e1);
-        s_score[g][lane] = e0;
-        s_score[g][lane + 64] = e1;
+        constexpr int PER_LANE = kAttnChunk / kWave;
+        float sc[PER_LANE];
+        float m = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < PER_LANE; u++) {
+            sc[u] = s_score[g][lane + u * kWave];
+            m = fmaxf(m, sc[u]);
+        }
+        m = wave_max(m);
+        float l = 0.0f;
+#pragma unroll
+        for (int u = 0; u < PER_LANE; u++) {
+            sc[u] = expf(sc[u] - m);
+            l += sc[u];
+            s_score[g][lane + u * kWave] = sc[u];
+        }
+        l = wave_sum(l);
         if (lane == 0) {
             ml_base[2 * g] = m;
             ml_base[2 * g + 1] = l;
@@ -262,71 +273,123 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
     }
 #pragma unroll
-    for (int it = 0; it < kAttnChunk / 16; it++) {
-        const int p = p0 + it * 16 + slot;
-        if (p < ctx) {
-            float vd[8];
-            unpack8(*reinterpret_cast<const uint4*>(v_cache + p * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub), vd);
+    for (int it = 0; it < ITERS; it++) {
+        // rows past the context carry weight 0; their (arbitrary) contents are zeroed so that a stray
+        // NaN or infinity cannot leak through 0 * x
+        const bool live = p0 + it * 16 + slot < ctx;
+        float vd[8];
+        unpack8(live ? make_uint4(vraw[it].x, vraw[it].y, vraw[it].z, vraw[it].w) : make_uint4(0u, 0u, 0u, 0u), vd);
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                const float wgt = s_score[g][it * 16 + slot];
+        for (int g = 0; g < G; g++) {
+            const float wgt = s_score[g][it * 16 + slot];
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[g][i] = __builtin_fmaf(wgt, vd[i], acc[g][i]);
-            }
+            for (int i = 0; i < 8; i++) acc[g][i] = __builtin_fmaf(wgt, vd[i], acc[g][i]);
         }
     }
-    // the four position slots of a wave meet through lane exchanges, the four waves through LDS
+    // the sixteen position slots meet in LDS, at most four heads at a time
+    constexpr int GH = G < kAccHeads ? G : kAccHeads;
 #pragma unroll
-    for (int g = 0; g < G; g++) {
+    for (int g0 = 0; g0 < G; g0 += GH) {
+        if (g0 > 0) __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            acc[g][i] += __shfl_xor(acc[g][i], 16, kWave);
-            acc[g][i] += __shfl_xor(acc[g][i], 32, kWave);
+        for (int g = 0; g < GH; g++) {
+            float4* dst = reinterpret_cast<float4*>(&s_acc[slot][g][8 * sub]);
+            dst[0] = make_float4(acc[g0 + g][0], acc[g0 + g][1], acc[g0 + g][2], acc[g0 + g][3]);
+            dst[1] = make_float4(acc[g0 + g][4], acc[g0 + g][5], acc[g0 + g][6], acc[g0 + g][7]);
         }
-        if (tid % kWave < 16) {
-            float4* dst = reinterpret_cast<float4*>(&s_acc[tid / kWave][g][8 * sub]);
-            dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-            dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
-        }
-    }
-    __syncthreads();
-    for (int o = tid; o < G * kHeadDim; o += kAttnThreads) {
-        const int g = o / kHeadDim;
-        const int d = o % kHeadDim;
-        float sum = 0.0f;
+        __syncthreads();
 #pragma unroll
-        for (int wv = 0; wv < kAttnThreads / kWave; wv++) sum += s_acc[wv][g][d];
-        out_base[o] = sum;
+        for (int o = tid; o < GH * kHeadDim; o += kAttnThreads) {
+            const int g = o / kHeadDim;
+            const int d = o % kHeadDim;
+            float part[kAttnSlots];
+#pragma unroll
+            for (int sl = 0; sl < kAttnSlots; sl++) part[sl] = s_acc[sl][g][d];
+            float sum = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < kAttnSlots; sl++) sum += part[sl];
+            out_base[g0 * kHeadDim + o] = sum;
+        }
     }
 }
 
+constexpr int kMergeParts = 4;  // chunk subsets summed side by side
+constexpr int kMergeThreads = kHeadDim * kMergeParts;
+
 template <int G>
-__global__ __launch_bounds__(kWave) void attn_decode_stage2(const float* __restrict__ part_out,
-                                                            const float* __restrict__ part_ml,
-                                                            uint16_t* __restrict__ out, int nchunks) {
+__global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float* __restrict__ part_out,
+                                                                    const float* __restrict__ part_ml,
+                                                                    uint16_t* __restrict__ out, int nchunks) {
+    extern __shared__ float s_factor[];  // nchunks rescaling factors exp(m_c - m)
+    __shared__ float s_red[kMergeThreads / kWave];
+    __shared__ float s_part[kMergeParts][kHeadDim];
     const int head = blockIdx.x;  // query head
     const int kvh = head / G;
     const int g = head % G;
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
     const float* ml = part_ml + static_cast<size_t>(kvh) * nchunks * G * 2;
+
+    // chunk maxima and sums, one chunk per thread at a time; both loads go out together
+    float mc_keep = -INFINITY, lc_keep = 0.0f;  // the thread's first chunk stays in registers
     float m = -INFINITY;
-    for (int c = lane; c < nchunks; c += kWave) m = fmaxf(m, ml[(static_cast<size_t>(c) * G + g) * 2]);
-    m = wave_max(m);
-    float l = 0.0f;
-    float a0 = 0.0f, a1 = 0.0f;  // dims lane and lane + 64
-    for (int c = 0; c < nchunks; c++) {
+    for (int c = tid; c < nchunks; c += kMergeThreads) {
         const float mc = ml[(static_cast<size_t>(c) * G + g) * 2];
         const float lc = ml[(static_cast<size_t>(c) * G + g) * 2 + 1];
-        if (lc == 0.0f) continue;  // chunk past the context
-        const float f = expf(mc - m);
-        l += lc * f;
-        const float* po = part_out + ((static_cast<size_t>(kvh) * nchunks + c) * G + g) * kHeadDim;
-        a0 += po[lane] * f;
-        a1 += po[lane + 64] * f;
+        if (c == tid) {
+            mc_keep = mc;
+            lc_keep = lc;
+        }
+        m = fmaxf(m, mc);
     }
-    const float inv = 1.0f / l;
-    out[static_cast<size_t>(head) * kHeadDim + lane] = f32_to_bf16(a0 * inv);
-    out[static_cast<size_t>(head) * kHeadDim + lane + 64] = f32_to_bf16(a1 * inv);
+    m = wave_max(m);
+    if (tid % kWave == 0) s_red[tid / kWave] = m;
+    __syncthreads();
+    m = s_red[0];
+#pragma unroll
+    for (int w = 1; w < kMergeThreads / kWave; w++) m = fmaxf(m, s_red[w]);
+    __syncthreads();
+    float l = 0.0f;
+    for (int c = tid; c < nchunks; c += kMergeThreads) {
+        const float mc = c == tid ? mc_keep : ml[(static_cast<size_t>(c) * G + g) * 2];
+        const float lc = c == tid ? lc_keep : ml[(static_cast<size_t>(c) * G + g) * 2 + 1];
+        const float f = lc > 0.0f ? expf(mc - m) : 0.0f;  // chunks past the context have lc == 0
+        s_factor[c] = f;
+        l += lc * f;
+    }
+    l = wave_sum(l);
+    if (tid % kWave == 0) s_red[tid / kWave] = l;
+    __syncthreads();
+    l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kMergeThreads / kWave; w++) l += s_red[w];
+
+    // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...; eight loads in flight
+    const int d = tid % kHeadDim;
+    const int part = tid / kHeadDim;
+    const float* po = part_out + (static_cast<size_t>(kvh) * nchunks * G + g) * kHeadDim + d;
+    const size_t cstride = static_cast<size_t>(G) * kHeadDim;
+    float acc = 0.0f;
+    for (int c0 = part; c0 < nchunks; c0 += 8 * kMergeParts) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int c = c0 + u * kMergeParts;
+            v[u] = (c < nchunks && s_factor[c] > 0.0f) ? po[c * cstride] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int c = c0 + u * kMergeParts;
+            if (c < nchunks) acc = __builtin_fmaf(v[u], s_factor[c], acc);
+        }
+    }
+    s_part[part][d] = acc;
+    __syncthreads();
+    if (part == 0) {
+        float total = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kMergeParts; q++) total += s_part[q][d];
+        out[static_cast<size_t>(head) * kHeadDim + d] = f32_to_bf16(total / l);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -381,13 +444,34 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* 
     __shared__ int s_idx[kArgmaxThreads / kWave];
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += kArgmaxThreads) {
-        const float v = bf16_to_f32(x[i]);
-        if (v > best) {  // ascending i per thread: the first maximum wins; NaN never compares greater
+    auto consider = [&](float v, int i) {
+        // strictly greater, or equal with a smaller index: the first maximum wins; NaN never wins
+        if (v > best || (v == best && i < best_i)) {
             best = v;
             best_i = i;
         }
+    };
+    const bool wide = (reinterpret_cast<uintptr_t>(x) % 16) == 0;
+    const int chunks = wide ? n / 8 : 0;
+    for (int c0 = threadIdx.x; c0 < chunks; c0 += 4 * kArgmaxThreads) {
+        uint4 raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int c = c0 + u * kArgmaxThreads;
+            raw[u] = c < chunks ? reinterpret_cast<const uint4*>(x)[c] : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int c = c0 + u * kArgmaxThreads;
+            if (c < chunks) {
+                float v[8];
+                unpack8(raw[u], v);
+#pragma unroll
+                for (int i = 0; i < 8; i++) consider(v[i], 8 * c + i);
+            }
+        }
     }
+    for (int i = 8 * chunks + threadIdx.x; i < n; i += kArgmaxThreads) consider(bf16_to_f32(x[i]), i);
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(best, off, kWave);
@@ -480,12 +564,12 @@ extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, c
     float* part_ml = part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
     const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
     hipStream_t s = kx::as_stream(stream);
-    dim3 grid1(n_kv_heads, nchunks);
+    dim3 grid1(nchunks, n_kv_heads);
 #define KX_ATTN(GG)                                                                                           \
     hipLaunchKernelGGL((kx::attn_decode_stage1<GG>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache, v_cache, \
-                       part_out, part_ml, n_kv_heads, pos, nchunks, scale);                                    \
-    hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kWave), 0, s, part_out, part_ml,  \
-                       out, nchunks)
+                       part_out, part_ml, n_kv_heads, pos, nchunks, max_positions, scale);                                    \
+    hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kMergeThreads),               \
+                       nchunks * sizeof(float), s, part_out, part_ml, out, nchunks)
     if (G == 1) { KX_ATTN(1); } else if (G == 2) { KX_ATTN(2); } else if (G == 4) { KX_ATTN(4); } else { KX_ATTN(8); }
 #undef KX_ATTN
     return kx::launch_status();
