@@ -40,6 +40,7 @@ extern "C" {
 #define KX_ERR_BAD_SHAPE (-2)      /* M/K/N/group outside what the kernels accept */
 #define KX_ERR_WORKSPACE (-3)      /* workspace missing or smaller than kx_gemv_*_workspace_bytes */
 #define KX_ERR_ALIGNMENT (-4)      /* a pointer is not aligned as documented */
+#define KX_ERR_ALIAS (-5)          /* an output overlaps an input that other workgroups still read */
 
 #define KX_MAX_BATCH 16            /* largest M the GEMV entry points take */
 
@@ -84,6 +85,33 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
  * 2 = the MFMA kernel wherever the group size allows.  Process-wide, not thread-safe.
  * Reference counterpart: none. */
 int kx_set_awq_kernel_policy(int policy);
+
+/* ------------------------------------------------------------------------------------------
+ * The same GEMV with the activations produced on the way in, for the decode step (one launch
+ * instead of two; built for M = 1, correct for M <= KX_MAX_BATCH, always the vector kernel).
+ * Rounding points are those of the stand-alone kernels further down, so each call returns what
+ * the two separate calls return (bitwise for kx_gemv_awq_swiglu_bf16 against the vector kernel).
+ *
+ *   kx_gemv_awq_swiglu_bf16:  x[m,k] = bf16( bf16(silu(gate[m,k])) * up[m,k] ),  y = x W
+ *       gate, up bf16, rows act_ld elements apart (act_ld >= K; halves of one [M, 2K] tensor or two
+ *       tensors), 2-byte aligned.
+ *   kx_gemv_awq_addnorm_bf16: r = bf16(residual + delta)   (delta may be null: r = residual)
+ *                             x = gain * bf16(r * rsqrt(mean_k(r^2) + eps)),  y = x W
+ *       residual, delta bf16 [M,K] (16-byte aligned), gain bf16 [K]; r is written to residual_out
+ *       [M,K] when that is not null.  residual_out must differ from residual and delta
+ *       (KX_ERR_ALIAS): every workgroup reads the whole incoming row.  K <= 8192.
+ * Replaces: LayerSwiGLU + LayerMatmul, resp. LayerAdd + LayerRMSNorm + LayerMatmul, executed back
+ * to back (slots kuiper/include/op/layer.h:8-20; none of the three is implemented in the reference).
+ * ------------------------------------------------------------------------------------------ */
+int kx_gemv_awq_swiglu_bf16(const uint16_t* gate, const uint16_t* up, int32_t act_ld,
+                            const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
+                            uint16_t* y, int32_t M, int32_t K, int32_t N, int32_t group_size,
+                            void* workspace, size_t workspace_bytes, void* stream);
+int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t* delta, const uint16_t* gain,
+                             float eps, uint16_t* residual_out, const int32_t* qweight,
+                             const uint16_t* scales, const int32_t* qzeros, uint16_t* y, int32_t M,
+                             int32_t K, int32_t N, int32_t group_size, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * BF16 GEMV fallback (non-quantised layers, lm_head):   y[m,n] = sum_k x[m,k] * W[n,k]

@@ -23,6 +23,9 @@ SIGNATURES = {
     "kx_gemv_awq_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_set_awq_kernel_policy": (ctypes.c_int, [ctypes.c_int]),
     "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_gemv_awq_swiglu_bf16": (ctypes.c_int, [_P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_gemv_awq_addnorm_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I32, _I32,
+                                                _I32, _I32, _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "kx_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
     "kx_add_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
@@ -102,6 +105,29 @@ def gemv_awq_bf16(x, qweight, scales, qzeros, y, group_size, workspace):
     _check(load().kx_gemv_awq_bf16(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
                                    M, K, N, group_size, _ptr(workspace),
                                    0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_awq_swiglu_bf16(gate, up, qweight, scales, qzeros, y, group_size, workspace):
+    """y = (bf16(bf16(silu(gate)) * up)) W; gate and up are bf16 [M,K] views that share a row stride."""
+    M, K = gate.shape
+    N = y.shape[-1]
+    if gate.stride(0) != up.stride(0) or gate.stride(1) != 1 or up.stride(1) != 1:
+        raise ValueError("gate and up must be row views with one common row stride")
+    _check(load().kx_gemv_awq_swiglu_bf16(_ptr(gate), _ptr(up), gate.stride(0), _ptr(qweight), _ptr(scales),
+                                          _ptr(qzeros), _ptr(y), M, K, N, group_size, _ptr(workspace),
+                                          0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_awq_addnorm_bf16(residual, delta, gain, eps, residual_out, qweight, scales, qzeros, y, group_size,
+                          workspace):
+    """r = bf16(residual + delta) (delta may be None), y = (gain * bf16(r * rsqrt(mean r^2 + eps))) W;
+    r goes to residual_out (may be None, must not be residual or delta)."""
+    M, K = residual.shape
+    N = y.shape[-1]
+    _check(load().kx_gemv_awq_addnorm_bf16(_ptr(residual), _ptr(delta), _ptr(gain), eps, _ptr(residual_out),
+                                           _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y), M, K, N,
+                                           group_size, _ptr(workspace),
+                                           0 if workspace is None else workspace.numel(), _stream()))
 
 
 def set_awq_kernel_policy(policy):

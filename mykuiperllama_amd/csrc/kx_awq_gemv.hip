@@ -91,6 +91,61 @@ void launch_mb(const AwqPlan& p, const uint16_t* x, const int32_t* qweight, cons
 #undef KX_ARGS
 }
 
+// Launches with an activation prologue are built for the decode step (M = 1); larger M is served
+// two activation rows per workgroup.
+inline AwqPlan make_fused_plan(int M, int K, int N) {
+    AwqPlan p = make_valu_plan(M, K, N);
+    p.mb = M >= 2 ? 2 : 1;
+    p.mtiles = (M + p.mb - 1) / p.mb;
+    return p;
+}
+
+template <int PRO>
+void launch_fused(const AwqPlan& p, const FusedInput& fi, const int32_t* qweight, const uint16_t* scales,
+                  const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters, int M, int K,
+                  int N, int group, hipStream_t stream) {
+#define KX_ARGS nullptr, qweight, scales, qzeros, y, partials, counters, M, K, N, group, p.coltiles, p.ktiles, p.mtiles, stream, fi
+#define KX_BY_MB(W, R)                                                  \
+    do {                                                                \
+        if (p.mb == 1) launch_awq_gemv<W, R, 1, PRO>(KX_ARGS);          \
+        else launch_awq_gemv<W, R, 2, PRO>(KX_ARGS);                    \
+    } while (0)
+    if (p.waves == 8) KX_BY_MB(8, 16);
+    else if (p.rt == 16) KX_BY_MB(4, 16);
+    else KX_BY_MB(4, 8);
+#undef KX_BY_MB
+#undef KX_ARGS
+}
+
+// Checks shared by every AWQ entry point; `x` stands for whichever tensors feed the activations.
+inline int check_awq_weights(const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
+                             const uint16_t* y, int M, int K, int N, int group_size) {
+    if (!qweight || !scales || !qzeros || !y) return KX_ERR_NULL_POINTER;
+    if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8 || (N % 8) != 0) return KX_ERR_BAD_SHAPE;
+    if (group_size < 32 || (group_size % 32) != 0 || (K % group_size) != 0) return KX_ERR_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(scales) % 16 || reinterpret_cast<uintptr_t>(qweight) % 4 ||
+        reinterpret_cast<uintptr_t>(qzeros) % 4 || reinterpret_cast<uintptr_t>(y) % 8) {
+        return KX_ERR_ALIGNMENT;
+    }
+    return KX_OK;
+}
+
+// Splits the workspace into counters and partial sums when the plan shares column tiles.
+inline int resolve_workspace(const AwqPlan& p, int M, int N, void* workspace, size_t workspace_bytes,
+                             float** partials, uint32_t** counters) {
+    *partials = nullptr;
+    *counters = nullptr;
+    if (p.ktiles <= 1) return KX_OK;
+    if (!workspace) return KX_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) % 256) return KX_ERR_ALIGNMENT;
+    const size_t need = kCounterBytes + static_cast<size_t>(p.ktiles) * M * N * sizeof(float);
+    if (workspace_bytes < need) return KX_ERR_WORKSPACE;
+    if (p.coltiles * p.mtiles > kMaxTiles) return KX_ERR_BAD_SHAPE;
+    *counters = static_cast<uint32_t*>(workspace);
+    *partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kCounterBytes);
+    return KX_OK;
+}
+
 __global__ void fill_zero_u32(uint32_t* p, size_t n) {
     size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -129,26 +184,15 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
                                 const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
                                 int32_t group_size, void* workspace, size_t workspace_bytes,
                                 void* stream) {
-    if (!x || !qweight || !scales || !qzeros || !y) return KX_ERR_NULL_POINTER;
-    if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8 || (N % 8) != 0) return KX_ERR_BAD_SHAPE;
-    if (group_size < 32 || (group_size % 32) != 0 || (K % group_size) != 0) return KX_ERR_BAD_SHAPE;
-    if (reinterpret_cast<uintptr_t>(scales) % 16 || reinterpret_cast<uintptr_t>(x) % 16 ||
-        reinterpret_cast<uintptr_t>(qweight) % 4 || reinterpret_cast<uintptr_t>(qzeros) % 4 ||
-        reinterpret_cast<uintptr_t>(y) % 8) {
-        return KX_ERR_ALIGNMENT;
-    }
+    if (!x) return KX_ERR_NULL_POINTER;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    if (reinterpret_cast<uintptr_t>(x) % 16) return KX_ERR_ALIGNMENT;
     kx::AwqPlan p = kx::make_plan(M, K, N, group_size);
     float* partials = nullptr;
     uint32_t* counters = nullptr;
-    if (p.ktiles > 1) {
-        if (!workspace) return KX_ERR_WORKSPACE;
-        if (reinterpret_cast<uintptr_t>(workspace) % 256) return KX_ERR_ALIGNMENT;
-        size_t need = kx::kCounterBytes + static_cast<size_t>(p.ktiles) * M * N * sizeof(float);
-        if (workspace_bytes < need) return KX_ERR_WORKSPACE;
-        if (p.coltiles * p.mtiles > kx::kMaxTiles) return KX_ERR_BAD_SHAPE;
-        counters = static_cast<uint32_t*>(workspace);
-        partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kx::kCounterBytes);
-    }
+    rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
     hipStream_t s = kx::as_stream(stream);
     if (p.mfma) {
         int group_shift = 0;
@@ -177,5 +221,62 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
         kx::launch_mb<4, 8>(KX_ARGS);
     }
 #undef KX_ARGS
+    return kx::launch_status();
+}
+
+extern "C" int kx_gemv_awq_swiglu_bf16(const uint16_t* gate, const uint16_t* up, int32_t act_ld,
+                                       const int32_t* qweight, const uint16_t* scales,
+                                       const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K,
+                                       int32_t N, int32_t group_size, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+    if (!gate || !up) return KX_ERR_NULL_POINTER;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    if (act_ld < K) return KX_ERR_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(gate) % 2 || reinterpret_cast<uintptr_t>(up) % 2) return KX_ERR_ALIGNMENT;
+    const kx::AwqPlan p = kx::make_fused_plan(M, K, N);
+    float* partials = nullptr;
+    uint32_t* counters = nullptr;
+    rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
+    kx::FusedInput fi{};
+    fi.a = gate;
+    fi.b = up;
+    fi.ld = act_ld;
+    kx::launch_fused<kx::kProSwiGLU>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N, group_size,
+                                     kx::as_stream(stream));
+    return kx::launch_status();
+}
+
+extern "C" int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t* delta, const uint16_t* gain,
+                                        float eps, uint16_t* residual_out, const int32_t* qweight,
+                                        const uint16_t* scales, const int32_t* qzeros, uint16_t* y,
+                                        int32_t M, int32_t K, int32_t N, int32_t group_size,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+    if (!residual || !gain) return KX_ERR_NULL_POINTER;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    if (reinterpret_cast<uintptr_t>(residual) % 16 || reinterpret_cast<uintptr_t>(delta) % 16 ||
+        reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
+        return KX_ERR_ALIGNMENT;
+    }
+    // every workgroup reads the whole incoming row while the first column tile writes the outgoing one
+    if (residual_out == residual || (residual_out && residual_out == delta)) return KX_ERR_ALIAS;
+    const kx::AwqPlan p = kx::make_fused_plan(M, K, N);
+    // a thread holds kNormChunks 16-byte pieces of the row for the sum of squares
+    if ((K >> 3) > kx::kNormChunks * p.waves * kx::kWave) return KX_ERR_BAD_SHAPE;
+    float* partials = nullptr;
+    uint32_t* counters = nullptr;
+    rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
+    kx::FusedInput fi{};
+    fi.a = residual;
+    fi.b = delta;
+    fi.gain = gain;
+    fi.r_out = residual_out;
+    fi.ld = K;
+    fi.eps = eps;
+    kx::launch_fused<kx::kProAddNorm>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N, group_size,
+                                      kx::as_stream(stream));
     return kx::launch_status();
 }

@@ -56,17 +56,64 @@ __device__ __forceinline__ void unpack_codes(uint32_t w, float (&q)[8]) {
     q[order_of(7)] = d.y;
 }
 
-template <int WAVES, int RT, int MB>
+// Activations may be produced on the way in instead of being read as a finished bf16 row
+// (PRO below); the producing arithmetic and its rounding points are those of the stand-alone
+// kernels, so a fused launch returns what the separate launches would.
+constexpr int kProNone = 0;     // x is a bf16 [M, K] tensor
+constexpr int kProSwiGLU = 1;   // x[m,k] = bf16( bf16(silu(a[m,k])) * b[m,k] )
+constexpr int kProAddNorm = 2;  // r = bf16(a + b) (b optional), x = gain * bf16(r * rsqrt(mean(r^2) + eps))
+constexpr int kNormChunks = 2;  // 16-byte pieces of a row a thread holds for the sum of squares
+
+struct FusedInput {
+    const uint16_t* a;     // gate, or the residual stream
+    const uint16_t* b;     // up, or the delta to add to the residual stream (may be null)
+    const uint16_t* gain;  // norm gain [K]
+    uint16_t* r_out;       // where the updated residual stream goes (may be null); must not alias a
+    int ld;                // elements between consecutive activation rows of a and b
+    float eps;
+};
+
+constexpr float kCodeOffset = 16.0f;
+
+// Two bf16 16.0 in a register whose value the compiler cannot see, so that (v & mask) | magic
+// selects as one v_and_or_b32 (a literal and a register) instead of v_and + v_or.
+__device__ __forceinline__ uint32_t opaque_bf16_pair_of_16() {
+    uint32_t out;
+    asm volatile("v_mov_b32 %0, 0x41804180" : "=v"(out));
+    return out;
+}
+
+// codes at bits 3..6 of each half -> bf16 pair (16 + q_lo, 16 + q_hi)
+__device__ __forceinline__ uint32_t code_pair_plus16(uint32_t v, uint32_t magic) {
+    return (v & 0x00780078u) | magic;
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// a.x * b.x + a.y * b.y + c in fp32, operands as packed bf16 pairs
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    bf16x2_t va, vb;
+    __builtin_memcpy(&va, &a, 4);
+    __builtin_memcpy(&vb, &b, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(va, vb, c, false);
+}
+
+template <int WAVES, int RT, int MB, int PRO>
 __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group, int coltiles, int ktiles) {
+    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi) {
     constexpr int SLOTS = WAVES * kSlotsPerWave;
     constexpr int KB = SLOTS * RT;
+    constexpr int THREADS = WAVES * kWave;
+    constexpr bool STAGED = PRO != kProNone;
     static_assert(RT % 8 == 0, "a lane reads its activations in 16-byte pieces");
+    static_assert(KB <= THREADS, "one staging thread per row of the workgroup's K range");
 
     __shared__ __attribute__((aligned(16))) float red[WAVES][kTileCols];
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? MB : 1][STAGED ? KB : 8];  // staged activations, bf16
+    __shared__ float s_ss[PRO == kProAddNorm ? MB : 1][WAVES];
 
     const int tid = threadIdx.x;
     const int ct = blockIdx.x % coltiles;
@@ -87,58 +134,172 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         for (int c = 0; c < 8; c++) acc[m][c] = 0.0f;
     }
 
-    if (active) {
-        // Small, cache-resident operands first, then every weight load of this lane, all of them
-        // issued before anything is consumed: loads return in order, so the arithmetic on row r
-        // can start while rows r+1.. are still in flight.
-        const int g = k0 / group;
-        const uint32_t zw = qzeros[static_cast<size_t>(g) * nw + wcg];
-        const uint4 sraw = *reinterpret_cast<const uint4*>(scales + static_cast<size_t>(g) * N + 8 * wcg);
-        uint4 xraw[MB][RT / 8];
+    // Operands of the activation prologue go out first: loads return in order, and the prologue
+    // should run while the weights are still on their way.  Thread t produces row kt*KB + t.
+    // Addresses are clamped instead of guarded so that the loads are straight-line code and all in
+    // flight together; what a clamped load returns is masked where it is used.
+    const int krow = kt * KB + tid;
+    const bool stager = STAGED && tid < KB && krow < K;
+    const bool has_b = PRO == kProSwiGLU || fi.b != nullptr;
+    const uint16_t* b_src = has_b ? fi.b : fi.a;  // without a delta the second operand is read and ignored
+    uint16_t own_a[MB], own_b[MB], own_gain = 0;
+    uint4 row_a[PRO == kProAddNorm ? MB : 1][kNormChunks], row_b[PRO == kProAddNorm ? MB : 1][kNormChunks];
+    if constexpr (STAGED) {
+        const int krow_c = krow < K ? krow : K - 1;
 #pragma unroll
         for (int m = 0; m < MB; m++) {
+            const int mrow = m0 + m < M ? m0 + m : M - 1;
+            const size_t at = static_cast<size_t>(mrow) * fi.ld + krow_c;
+            own_a[m] = fi.a[at];
+            own_b[m] = b_src[at];
+        }
+        if constexpr (PRO == kProAddNorm) own_gain = fi.gain[krow_c];
+    }
+    if constexpr (PRO == kProAddNorm) {
+        const int last_chunk = (K >> 3) - 1;
 #pragma unroll
-            for (int r8 = 0; r8 < RT / 8; r8++) {
-                xraw[m][r8] = (m0 + m < M)
-                    ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + m) * K + k0 + 8 * r8)
-                    : make_uint4(0u, 0u, 0u, 0u);
+        for (int m = 0; m < MB; m++) {
+            const int mrow = m0 + m < M ? m0 + m : M - 1;
+#pragma unroll
+            for (int j = 0; j < kNormChunks; j++) {
+                const int c = tid + j * THREADS;
+                const size_t at = static_cast<size_t>(mrow) * fi.ld + 8 * (c < last_chunk ? c : last_chunk);
+                row_a[m][j] = *reinterpret_cast<const uint4*>(fi.a + at);
+                row_b[m][j] = *reinterpret_cast<const uint4*>(b_src + at);
             }
         }
-        uint32_t w[RT];
-        const uint32_t* wp = qweight + static_cast<size_t>(k0) * nw + wcg;
+    }
+
+    // Small, cache-resident operands first, then every weight load of this lane, all of them
+    // issued before anything is consumed: loads return in order, so the arithmetic on row r
+    // can start while rows r+1.. are still in flight.
+    // With a prologue the loads are not guarded either: a branch around them would make the wait
+    // for the prologue's operands a wait for the weights as well.  Lanes outside the matrix read a
+    // clamped address and take no part in the arithmetic.
+    uint32_t zw = 0;
+    uint4 sraw = make_uint4(0u, 0u, 0u, 0u);
+    uint4 xraw[MB][RT / 8];
+    uint32_t w[RT];
+    if (STAGED || active) {
+        const int ld_wcg = STAGED ? (wcg < nw ? wcg : nw - 1) : wcg;
+        const int ld_k0 = STAGED ? (k0 < K ? k0 : K - RT) : k0;
+        const int g = ld_k0 / group;
+        zw = qzeros[static_cast<size_t>(g) * nw + ld_wcg];
+        sraw = *reinterpret_cast<const uint4*>(scales + static_cast<size_t>(g) * N + 8 * ld_wcg);
+        if constexpr (!STAGED) {
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+#pragma unroll
+                for (int r8 = 0; r8 < RT / 8; r8++) {
+                    xraw[m][r8] = (m0 + m < M)
+                        ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + m) * K + k0 + 8 * r8)
+                        : make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+        }
+        const uint32_t* wp = qweight + static_cast<size_t>(ld_k0) * nw + ld_wcg;
 #pragma unroll
         for (int r = 0; r < RT; r++) {
             w[r] = __builtin_nontemporal_load(wp + static_cast<size_t>(r) * nw);
         }
         // keep the scheduler from sinking loads below the first use of an earlier one
         __builtin_amdgcn_sched_barrier(0);
+    }
 
+    if constexpr (PRO == kProSwiGLU) {
+        if (tid < KB) {
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+                const float gt = bf16_to_f32(own_a[m]);
+                const float act = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+                const uint16_t xv = f32_to_bf16(act * bf16_to_f32(own_b[m]));
+                s_x[m][tid] = (stager && m0 + m < M) ? xv : static_cast<uint16_t>(0);
+            }
+        }
+        lds_barrier();
+    }
+    if constexpr (PRO == kProAddNorm) {
+        // sum of squares of the whole updated row, in the order of the stand-alone norm kernel
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kNormChunks; j++) {
+                const uint32_t aw[4] = {row_a[m][j].x, row_a[m][j].y, row_a[m][j].z, row_a[m][j].w};
+                const uint32_t bw[4] = {row_b[m][j].x, row_b[m][j].y, row_b[m][j].z, row_b[m][j].w};
+                const bool valid = tid + j * THREADS < (K >> 3);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float av = __uint_as_float((i & 1) ? (aw[i >> 1] & 0xffff0000u) : (aw[i >> 1] << 16));
+                    const float bv = __uint_as_float((i & 1) ? (bw[i >> 1] & 0xffff0000u) : (bw[i >> 1] << 16));
+                    // r = bf16(a + b); without a delta r = a, whose square a + 0 leaves unchanged
+                    const float r = bf16_to_f32(f32_to_bf16(av + (has_b ? bv : 0.0f)));
+                    ss += valid ? r * r : 0.0f;
+                }
+            }
+            ss = wave_sum(ss);
+            if (tid % kWave == 0) s_ss[m][tid / kWave] = ss;
+        }
+        lds_barrier();
+        if (tid < KB) {
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+                float total = 0.0f;
+#pragma unroll
+                for (int u = 0; u < WAVES; u++) total += s_ss[m][u];
+                const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + fi.eps);
+                const uint16_t sum_bits = f32_to_bf16(bf16_to_f32(own_a[m]) + bf16_to_f32(own_b[m]));
+                const uint16_t rbits = has_b ? sum_bits : own_a[m];
+                const float r = bf16_to_f32(rbits);
+                const float h = bf16_to_f32(own_gain) * bf16_to_f32(f32_to_bf16(r * inv));
+                const bool live = stager && m0 + m < M;
+                s_x[m][tid] = live ? f32_to_bf16(h) : static_cast<uint16_t>(0);
+                if (ct == 0 && live && fi.r_out) {
+                    fi.r_out[static_cast<size_t>(m0 + m) * K + krow] = rbits;
+                }
+            }
+        }
+        lds_barrier();
+    }
+
+    if (active) {
+        // Two rows at a time: the codes of rows k and k+1 of one column become a pair of bf16 numbers
+        // 16 + q (exponent of 16.0, the code in the top four mantissa bits), the activations of the two
+        // rows already lie in memory as such a pair, and one dot-product instruction does both
+        // multiply-adds in fp32.  The offset is taken out again with the zero point:
+        //   sum_k x (q - z) = sum_k x (16 + q)  -  (16 + z) sum_k x
+        const uint32_t magic = opaque_bf16_pair_of_16();
+        const uint32_t ones = 0x3F803F80u;  // bf16 (1, 1)
         float xsum[MB];
 #pragma unroll
         for (int m = 0; m < MB; m++) xsum[m] = 0.0f;
 
 #pragma unroll
-        for (int r8 = 0; r8 < RT; r8 += 8) {
-            float xs[MB][8];
+        for (int rp = 0; rp < RT / 2; rp++) {
+            uint32_t xp[MB];
 #pragma unroll
             for (int m = 0; m < MB; m++) {
-                const uint4 xr = xraw[m][r8 / 8];
-                const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
-#pragma unroll
-                for (int r = 0; r < 8; r++) {
-                    const uint32_t bits = (r & 1) ? (xw[r >> 1] & 0xffff0000u) : (xw[r >> 1] << 16);
-                    xs[m][r] = __uint_as_float(bits);
-                    xsum[m] += xs[m][r];
+                if constexpr (STAGED) {
+                    xp[m] = *reinterpret_cast<const uint32_t*>(&s_x[m][slot * RT + 2 * rp]);
+                } else {
+                    const uint4 xr = xraw[m][rp / 4];
+                    const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
+                    xp[m] = xw[rp % 4];
                 }
+                xsum[m] = dot2_bf16(xp[m], ones, xsum[m]);
             }
+            const uint32_t wa = w[2 * rp], wb = w[2 * rp + 1];
+            const uint32_t lo = __builtin_amdgcn_perm(wb, wa, 0x05040100u);  // nibbles 0..3 of both rows
+            const uint32_t hi = __builtin_amdgcn_perm(wb, wa, 0x07060302u);  // nibbles 4..7
 #pragma unroll
-            for (int r = 0; r < 8; r++) {
-                float q[8];
-                unpack_codes(w[r8 + r], q);
+            for (int i = 0; i < 4; i++) {
+                // nibble i sits at bits 4i of each half and goes to bits 3..6
+                const uint32_t plo = code_pair_plus16(i == 0 ? lo << 3 : lo >> (4 * i - 3), magic);
+                const uint32_t phi = code_pair_plus16(i == 0 ? hi << 3 : hi >> (4 * i - 3), magic);
 #pragma unroll
                 for (int m = 0; m < MB; m++) {
-#pragma unroll
-                    for (int c = 0; c < 8; c++) acc[m][c] = __builtin_fmaf(q[c], xs[m][r], acc[m][c]);
+                    acc[m][order_of(i)] = dot2_bf16(plo, xp[m], acc[m][order_of(i)]);
+                    acc[m][order_of(4 + i)] = dot2_bf16(phi, xp[m], acc[m][order_of(4 + i)]);
                 }
             }
         }
@@ -147,17 +308,14 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         float z[8];
         unpack_codes(zw, z);
         const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
-        float s[8];
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
-            s[c] = f16_bits_to_f32(bits) * kCodeScale;  // power of two: exact
-        }
+            const float sc = f16_bits_to_f32(bits);
+            const float zoff = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
 #pragma unroll
-        for (int m = 0; m < MB; m++) {
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-                acc[m][c] = s[c] * __builtin_fmaf(-z[c], xsum[m], acc[m][c]);
+            for (int m = 0; m < MB; m++) {
+                acc[m][c] = sc * __builtin_fmaf(-zoff, xsum[m], acc[m][c]);
             }
         }
     }
@@ -195,17 +353,17 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
                               &s_prev);
 }
 
-template <int WAVES, int RT, int MB>
+template <int WAVES, int RT, int MB, int PRO = kProNone>
 inline void launch_awq_gemv(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
                             const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
                             int M, int K, int N, int group, int coltiles, int ktiles, int mtiles,
-                            hipStream_t stream) {
+                            hipStream_t stream, const FusedInput& fi = FusedInput{}) {
     dim3 grid(coltiles * ktiles, mtiles, 1);
     dim3 block(WAVES * kWave, 1, 1);
-    hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB>), grid, block, 0, stream, x,
+    hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB, PRO>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group, coltiles, ktiles);
+                       group, coltiles, ktiles, fi);
 }
 
 }  // namespace kx

@@ -88,6 +88,14 @@ __device__ __forceinline__ float wave_max(float v) {
     return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
 }
 
+// Workgroup barrier for data that travels through LDS only: orders LDS accesses and leaves global
+// loads that are still in flight alone (a full __syncthreads() waits for those as well).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 inline hipStream_t as_stream(void* s) {
     return static_cast<hipStream_t>(s);
 }

@@ -12,6 +12,7 @@ extern "C" const char* kx_error_string(int code) {
         case KX_ERR_BAD_SHAPE: return "shape or group size not accepted by the kernels";
         case KX_ERR_WORKSPACE: return "workspace missing or too small (see kx_gemv_workspace_bytes)";
         case KX_ERR_ALIGNMENT: return "pointer not aligned as the interface requires";
+        case KX_ERR_ALIAS: return "an output overlaps an input that is still being read";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

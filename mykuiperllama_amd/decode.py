@@ -13,8 +13,12 @@ the usual pre-norm decoder with per-head QK-norm:
 q/k/v share one fused GEMV (N = (n_q + 2 n_kv) * 128) and gate/up another (N = 2 * intermediate): the
 packed tensors of the separate projections are concatenated along N when the weights are loaded
 (rows are laid end to end; the nibble order inside a word is untouched).  The residual add is fused
-into the next RMSNorm.  Every launch goes to torch's current stream, so a step can be captured in
-a HIP graph; token and position live in device memory for that reason.
+into the next RMSNorm, and by default (`fused=True`) both ride in the prologue of the GEMV that
+consumes the normalised row, as does SwiGLU in front of the down projection: seven launches per
+layer instead of ten.  The residual stream then alternates between two buffers, because a fused
+launch reads the whole incoming row in every workgroup while it writes the updated one.
+Every launch goes to torch's current stream, so a step can be captured in a HIP graph; token and
+position live in device memory for that reason.
 """
 from dataclasses import dataclass
 
@@ -96,6 +100,7 @@ class DecodeModel:
             return torch.zeros((1, n), dtype=bf, device="cuda")
 
         self.x = buf(c.hidden)
+        self.x2 = buf(c.hidden)
         self.h = buf(c.hidden)
         self.qkv = buf(c.qkv_out)
         self.q = buf(c.n_q * c.head_dim)
@@ -129,8 +134,10 @@ class DecodeModel:
     def _awq(self, x, w, y):
         capi.gemv_awq_bf16(x, w[0], w[1], w[2], y, self.cfg.group, self.gemv_ws)
 
-    def step(self, with_lm_head=True):
+    def step(self, with_lm_head=True, fused=True):
         """Enqueue one decode step on torch's current stream (no synchronisation)."""
+        if fused:
+            return self._step_fused(with_lm_head)
         c = self.cfg
         capi.embedding_bf16(self.embed, self.token, self.x)
         for li, L in enumerate(self.layers):
@@ -153,8 +160,32 @@ class DecodeModel:
             capi.gemv_bf16(self.h, self.lm_head, self.logits)
             capi.argmax_bf16(self.logits, self.next_token)
 
-    def launches_per_step(self, with_lm_head=True):
-        return 1 + self.cfg.layers * 10 + 1 + (2 if with_lm_head else 0)
+    def _step_fused(self, with_lm_head):
+        c = self.cfg
+        g, ws = c.group, self.gemv_ws
+        capi.embedding_bf16(self.embed, self.token, self.x)
+        xa, xb = self.x, self.x2
+        for li, L in enumerate(self.layers):
+            qw, sc, qz = L["qkv"]
+            capi.gemv_awq_addnorm_bf16(xa, None if li == 0 else self.down, L["in_norm"], c.eps, xb, qw, sc, qz,
+                                       self.qkv, g, ws)
+            capi.qk_norm_rope_bf16(self.qkv, L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
+                                   c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps)
+            capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
+                                  self.max_positions, self.attn_ws)
+            self._awq(self.attn, L["o"], self.o)
+            qw, sc, qz = L["gateup"]
+            capi.gemv_awq_addnorm_bf16(xb, self.o, L["post_norm"], c.eps, xa, qw, sc, qz, self.gu, g, ws)
+            qw, sc, qz = L["down"]
+            capi.gemv_awq_swiglu_bf16(self.gu[:, : c.intermediate], self.gu[:, c.intermediate:], qw, sc, qz,
+                                      self.down, g, ws)
+        capi.add_rmsnorm_bf16(xa, self.down, self.final_norm, self.h, c.eps)
+        if with_lm_head:
+            capi.gemv_bf16(self.h, self.lm_head, self.logits)
+            capi.argmax_bf16(self.logits, self.next_token)
+
+    def launches_per_step(self, with_lm_head=True, fused=True):
+        return 1 + self.cfg.layers * (7 if fused else 10) + 1 + (2 if with_lm_head else 0)
 
 
 def step_bytes(cfg, ctx, with_lm_head=True):

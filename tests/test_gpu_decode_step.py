@@ -125,7 +125,8 @@ class Reference:
         return x, logits
 
 
-def test_decode_steps_match_the_fp32_reference(torch, oracle):
+@pytest.mark.parametrize("fused", [True, False])
+def test_decode_steps_match_the_fp32_reference(torch, oracle, fused):
     from mykuiperllama_amd import decode
     cfg = decode.ModelConfig(**CFG)
     layers_np, layers_ref, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
@@ -138,7 +139,7 @@ def test_decode_steps_match_the_fp32_reference(torch, oracle):
     for stepno in range(4):
         pos = CTX + stepno
         model.set_input(token, pos)
-        model.step()
+        model.step(fused=fused)
         torch.cuda.synchronize()
         x_ref, logits_ref = ref.step(token, pos)
         got_logits = model.logits[0].cpu().float()
@@ -159,21 +160,38 @@ def test_decode_steps_match_the_fp32_reference(torch, oracle):
     assert agreed >= 1
 
 
-def test_step_is_capturable_in_a_graph_and_replays_identically(torch):
+def test_fused_and_separate_launches_give_the_same_step(torch):
+    """SwiGLU and add+RMSNorm in the GEMV prologue change nothing, bit for bit."""
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    model = decode.DecodeModel(cfg, MAXPOS)
+    model.prefill_cache_random(CTX)
+    results = []
+    for fused in (False, True):
+        model.set_input(9, CTX)
+        model.step(fused=fused)
+        torch.cuda.synchronize()
+        results.append((model.logits.clone(), model.x.clone(), model.k_cache[-1][CTX].clone()))
+    for a, b in zip(*results):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_step_is_capturable_in_a_graph_and_replays_identically(torch, fused):
     """A captured step replayed with the same inputs gives bitwise the same logits as eager."""
     from mykuiperllama_amd import decode
     cfg = decode.ModelConfig(**CFG)
     model = decode.DecodeModel(cfg, MAXPOS)
     model.prefill_cache_random(CTX)
     model.set_input(5, CTX)
-    model.step()
+    model.step(fused=fused)
     torch.cuda.synchronize()
     eager = model.logits.clone()
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            model.step()
+            model.step(fused=fused)
         for _ in range(3):
             model.logits.zero_()
             torch.cuda.synchronize()

@@ -1,0 +1,211 @@
+"""GPU parity of the AWQ GEMV entry points that produce their activations on the way in.
+
+Two independent checks per entry point:
+  * against the stand-alone kernels run back to back (SwiGLU or add+RMSNorm, then the GEMV on the
+    vector kernel): bitwise for the SwiGLU prologue and for the norm prologue on workgroups of eight
+    waves, whose sum of squares is added in the stand-alone kernel's order; otherwise the
+    normalised row may differ by an ulp in a few places and the tolerance of the GEMV applies;
+  * against the CPU oracle's fp64 GEMV fed with activations computed by torch in fp32 with the
+    same rounding points (relative L2 <= 1e-3 against the rounded result).
+"""
+import numpy as np
+import pytest
+
+from mykuiperllama_amd import synth
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_ROUNDED = 1e-3
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch as _t
+    assert _t.cuda.is_available(), "GPU tests need a visible MI355X"
+    return _t
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from mykuiperllama_amd import capi as _c
+    _c.load()
+    return _c
+
+
+@pytest.fixture(autouse=True)
+def vector_kernel_for_the_unfused_side(capi):
+    capi.set_awq_kernel_policy(1)
+    yield
+    capi.set_awq_kernel_policy(0)
+
+
+def weights(torch, name, M, K, N, group):
+    p = synth.make_awq_problem(name, M, K, N, group)
+    dev = (H.to_dev_i32(p["qweight"], torch), H.to_dev_f16(p["scales"], torch), H.to_dev_i32(p["qzeros"], torch))
+    return p, dev
+
+
+def oracle_check(oracle, torch, p, x_dev, y_dev):
+    x_bits = H.bf16_bits(x_dev, torch)
+    ref64 = oracle.gemv_awq_f64(x_bits, p["qweight"], p["scales"], p["qzeros"], p["group"])
+    ref_rounded = H.bf16_to_f64(oracle.f32_to_bf16(ref64.astype(np.float32)))
+    got = H.bf16_to_f64(H.bf16_bits(y_dev, torch))
+    assert np.isfinite(got).all()
+    assert H.rel_l2(got, ref_rounded) <= REL_L2_ROUNDED
+    assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
+
+
+SWIGLU_CASES = [
+    # M, K, N, group, gate and up as halves of one tensor?
+    (1, 12288, 4096, 128, True),    # Qwen3-8B down_proj
+    (1, 25600, 5120, 128, True),    # Qwen3-32B down_proj
+    (1, 256, 512, 128, False),
+    (1, 128, 264, 32, False),       # K below one full workgroup, ragged N
+    (1, 96, 40, 32, True),
+    (2, 1024, 2048, 128, True),
+    (3, 4096, 1024, 128, False),
+    (5, 2048, 512, 64, True),
+    (16, 512, 256, 128, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,group,halves", SWIGLU_CASES)
+def test_swiglu_prologue_equals_separate_launches(capi, torch, oracle, M, K, N, group, halves):
+    p, (qw, sc, qz) = weights(torch, f"fused_swiglu_{M}_{K}_{N}", M, K, N, group)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(K * 31 + N + M)
+    if halves:
+        gu = (torch.randn((M, 2 * K), device="cuda", generator=g) * 1.5).bfloat16()
+        gate, up = gu[:, :K], gu[:, K:]
+    else:
+        gate = (torch.randn((M, K), device="cuda", generator=g) * 1.5).bfloat16()
+        up = torch.randn((M, K), device="cuda", generator=g).bfloat16()
+    ws = capi.make_workspace(M, K, N)
+    act = torch.empty((M, K), dtype=torch.bfloat16, device="cuda")
+    y_sep = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    y_fused = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.swiglu_bf16(gate.contiguous(), up.contiguous(), act)
+    capi.gemv_awq_bf16(act, qw, sc, qz, y_sep, group, ws)
+    capi.gemv_awq_swiglu_bf16(gate, up, qw, sc, qz, y_fused, group, ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(H.bf16_bits(y_fused, torch), H.bf16_bits(y_sep, torch))
+    # activations recomputed by torch with the same rounding points feed the oracle
+    silu = torch.nn.functional.silu(gate.float()).bfloat16().float()
+    act_ref = (silu * up.float()).bfloat16()
+    # expf of the kernel and torch's sigmoid may round an activation differently once in a while
+    assert (act_ref.view(torch.int16).int() - act.view(torch.int16).int()).abs().max().item() <= 1
+    oracle_check(oracle, torch, p, act, y_fused)
+
+
+ADDNORM_CASES = [
+    # M, K, N, group, with delta, with residual_out
+    (1, 4096, 6144, 128, True, True),    # Qwen3-8B fused q/k/v
+    (1, 4096, 24576, 128, True, True),   # Qwen3-8B fused gate/up
+    (1, 5120, 10240, 128, True, True),   # Qwen3-32B fused q/k/v: two pieces of the row per thread
+    (1, 8192, 512, 128, True, False),
+    (1, 4096, 1024, 128, False, False),  # plain RMSNorm (first layer)
+    (1, 4096, 1024, 128, False, True),
+    (1, 256, 512, 32, True, True),
+    (1, 128, 264, 32, True, True),       # four waves per workgroup
+    (1, 64, 40, 32, True, True),
+    (2, 1024, 2048, 128, True, True),
+    (5, 2048, 520, 64, True, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,group,with_delta,with_out", ADDNORM_CASES)
+def test_addnorm_prologue_equals_separate_launches(capi, torch, oracle, M, K, N, group, with_delta, with_out):
+    eps = 1e-6
+    p, (qw, sc, qz) = weights(torch, f"fused_addnorm_{M}_{K}_{N}", M, K, N, group)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(K * 17 + N + M)
+    resid = (torch.randn((M, K), device="cuda", generator=g) * 2.0).bfloat16()
+    delta = torch.randn((M, K), device="cuda", generator=g).bfloat16() if with_delta else None
+    gain = (1 + 0.1 * torch.randn((K,), device="cuda", generator=g)).bfloat16()
+    ws = capi.make_workspace(M, K, N)
+
+    x_sep = resid.clone()
+    h_sep = torch.empty((M, K), dtype=torch.bfloat16, device="cuda")
+    y_sep = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    if with_delta:
+        capi.add_rmsnorm_bf16(x_sep, delta, gain, h_sep, eps)
+    else:
+        capi.rmsnorm_bf16(x_sep, gain, h_sep, eps)
+    capi.gemv_awq_bf16(h_sep, qw, sc, qz, y_sep, group, ws)
+
+    resid_before = resid.clone()
+    r_out = torch.full((M, K), float("nan"), dtype=torch.bfloat16, device="cuda") if with_out else None
+    y_fused = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_addnorm_bf16(resid, delta, gain, eps, r_out, qw, sc, qz, y_fused, group, ws)
+    torch.cuda.synchronize()
+
+    assert torch.equal(resid, resid_before), "the incoming residual stream is read only"
+    if with_out:
+        assert np.array_equal(H.bf16_bits(r_out, torch), H.bf16_bits(x_sep, torch))
+    if K >= 256:
+        assert np.array_equal(H.bf16_bits(y_fused, torch), H.bf16_bits(y_sep, torch))
+    else:
+        a, b = y_fused.float().cpu().numpy(), y_sep.float().cpu().numpy()
+        assert H.rel_l2(a, b) <= REL_L2_ROUNDED
+    # fp32 torch restatement of the prologue, then the oracle's GEMV
+    r = (resid.float() + delta.float()).bfloat16().float() if with_delta else resid.float()
+    inv = torch.rsqrt((r * r).mean(dim=-1, keepdim=True) + eps)
+    h_ref = (gain.float() * (r * inv).bfloat16().float()).bfloat16()
+    assert (h_ref.view(torch.int16).int() - h_sep.view(torch.int16).int()).abs().max().item() <= 1
+    oracle_check(oracle, torch, p, h_sep, y_fused)
+
+
+def test_fused_launches_are_deterministic_and_leave_the_workspace_reusable(capi, torch):
+    M, K, N, group = 1, 4096, 6144, 128
+    _, (qw, sc, qz) = weights(torch, "fused_repeat", M, K, N, group)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    resid = torch.randn((M, K), device="cuda", generator=g).bfloat16()
+    delta = torch.randn((M, K), device="cuda", generator=g).bfloat16()
+    gain = torch.ones((K,), device="cuda").bfloat16()
+    ws = capi.make_workspace(M, K, N)
+    outs = []
+    for _ in range(4):
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        r = torch.empty((M, K), dtype=torch.bfloat16, device="cuda")
+        capi.gemv_awq_addnorm_bf16(resid, delta, gain, 1e-6, r, qw, sc, qz, y, group, ws)
+        outs.append(y)
+    torch.cuda.synchronize()
+    for y in outs[1:]:
+        assert torch.equal(y.view(torch.int16), outs[0].view(torch.int16))
+
+
+def test_fused_entry_points_reject_bad_arguments(capi, torch):
+    M, K, N, group = 1, 1024, 512, 128
+    _, (qw, sc, qz) = weights(torch, "fused_bad", M, K, N, group)
+    x = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda")
+    gain = torch.ones((K,), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ws = capi.make_workspace(M, K, N)
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_addnorm_bf16(x, None, gain, 1e-6, x, qw, sc, qz, y, group, ws)  # in place
+    assert e.value.code == -5
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_addnorm_bf16(x, x, gain, 1e-6, None, qw, sc, qz, y, group, None)  # split K, no workspace
+    assert e.value.code == -3
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_addnorm_bf16(x, None, None, 1e-6, None, qw, sc, qz, y, group, ws)
+    assert e.value.code == -1
+    rc = capi.load().kx_gemv_awq_swiglu_bf16(x.data_ptr(), None, K, qw.data_ptr(), sc.data_ptr(), qz.data_ptr(),
+                                             y.data_ptr(), M, K, N, group, ws.data_ptr(), ws.numel(), None)
+    assert rc == -1  # up missing
+    rc = capi.load().kx_gemv_awq_swiglu_bf16(x.data_ptr(), x.data_ptr(), K - 8, qw.data_ptr(), sc.data_ptr(),
+                                             qz.data_ptr(), y.data_ptr(), M, K, N, group, ws.data_ptr(),
+                                             ws.numel(), None)
+    assert rc == -2  # rows closer together than they are long
+    # a row longer than the norm prologue holds in registers
+    Kbig = 8192 + 128
+    _, (qw2, sc2, qz2) = weights(torch, "fused_bad_big", 1, Kbig, 256, 128)
+    xb = torch.zeros((1, Kbig), dtype=torch.bfloat16, device="cuda")
+    gb = torch.ones((Kbig,), dtype=torch.bfloat16, device="cuda")
+    yb = torch.zeros((1, 256), dtype=torch.bfloat16, device="cuda")
+    wsb = capi.make_workspace(1, Kbig, 256)
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_addnorm_bf16(xb, None, gb, 1e-6, None, qw2, sc2, qz2, yb, 128, wsb)
+    assert e.value.code == -2
