@@ -276,7 +276,12 @@ extern "C" int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t
     fi.r_out = residual_out;
     fi.ld = K;
     fi.eps = eps;
-    kx::launch_fused<kx::kProAddNorm>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N, group_size,
-                                      kx::as_stream(stream));
+    if ((K >> 3) <= p.waves * kx::kWave) {
+        kx::launch_fused<kx::kProAddNorm>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N,
+                                          group_size, kx::as_stream(stream));
+    } else {
+        kx::launch_fused<kx::kProAddNormLong>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N,
+                                              group_size, kx::as_stream(stream));
+    }
     return kx::launch_status();
 }

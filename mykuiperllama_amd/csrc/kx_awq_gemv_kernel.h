@@ -62,7 +62,8 @@ __device__ __forceinline__ void unpack_codes(uint32_t w, float (&q)[8]) {
 constexpr int kProNone = 0;     // x is a bf16 [M, K] tensor
 constexpr int kProSwiGLU = 1;   // x[m,k] = bf16( bf16(silu(a[m,k])) * b[m,k] )
 constexpr int kProAddNorm = 2;  // r = bf16(a + b) (b optional), x = gain * bf16(r * rsqrt(mean(r^2) + eps))
-constexpr int kNormChunks = 2;  // 16-byte pieces of a row a thread holds for the sum of squares
+constexpr int kProAddNormLong = 3;  // the same for rows of more than eight elements per thread
+constexpr int kNormChunks = 2;  // most 16-byte pieces of a row a thread holds for the sum of squares
 
 struct FusedInput {
     const uint16_t* a;     // gate, or the residual stream
@@ -108,12 +109,14 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     constexpr int KB = SLOTS * RT;
     constexpr int THREADS = WAVES * kWave;
     constexpr bool STAGED = PRO != kProNone;
+    constexpr bool NORM = PRO == kProAddNorm || PRO == kProAddNormLong;
+    constexpr int NCH = PRO == kProAddNormLong ? kNormChunks : 1;
     static_assert(RT % 8 == 0, "a lane reads its activations in 16-byte pieces");
     static_assert(KB <= THREADS, "one staging thread per row of the workgroup's K range");
 
     __shared__ __attribute__((aligned(16))) float red[WAVES][kTileCols];
     __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? MB : 1][STAGED ? KB : 8];  // staged activations, bf16
-    __shared__ float s_ss[PRO == kProAddNorm ? MB : 1][WAVES];
+    __shared__ float s_ss[NORM ? MB : 1][WAVES];
 
     const int tid = threadIdx.x;
     const int ct = blockIdx.x % coltiles;
@@ -143,7 +146,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const bool has_b = PRO == kProSwiGLU || fi.b != nullptr;
     const uint16_t* b_src = has_b ? fi.b : fi.a;  // without a delta the second operand is read and ignored
     uint16_t own_a[MB], own_b[MB], own_gain = 0;
-    uint4 row_a[PRO == kProAddNorm ? MB : 1][kNormChunks], row_b[PRO == kProAddNorm ? MB : 1][kNormChunks];
+    uint4 row_a[NORM ? MB : 1][NCH], row_b[NORM ? MB : 1][NCH];
     if constexpr (STAGED) {
         const int krow_c = krow < K ? krow : K - 1;
 #pragma unroll
@@ -153,15 +156,15 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             own_a[m] = fi.a[at];
             own_b[m] = b_src[at];
         }
-        if constexpr (PRO == kProAddNorm) own_gain = fi.gain[krow_c];
+        if constexpr (NORM) own_gain = fi.gain[krow_c];
     }
-    if constexpr (PRO == kProAddNorm) {
+    if constexpr (NORM) {
         const int last_chunk = (K >> 3) - 1;
 #pragma unroll
         for (int m = 0; m < MB; m++) {
             const int mrow = m0 + m < M ? m0 + m : M - 1;
 #pragma unroll
-            for (int j = 0; j < kNormChunks; j++) {
+            for (int j = 0; j < NCH; j++) {
                 const int c = tid + j * THREADS;
                 const size_t at = static_cast<size_t>(mrow) * fi.ld + 8 * (c < last_chunk ? c : last_chunk);
                 row_a[m][j] = *reinterpret_cast<const uint4*>(fi.a + at);
@@ -218,13 +221,13 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
         lds_barrier();
     }
-    if constexpr (PRO == kProAddNorm) {
+    if constexpr (NORM) {
         // sum of squares of the whole updated row, in the order of the stand-alone norm kernel
 #pragma unroll
         for (int m = 0; m < MB; m++) {
             float ss = 0.0f;
 #pragma unroll
-            for (int j = 0; j < kNormChunks; j++) {
+            for (int j = 0; j < NCH; j++) {
                 const uint32_t aw[4] = {row_a[m][j].x, row_a[m][j].y, row_a[m][j].z, row_a[m][j].w};
                 const uint32_t bw[4] = {row_b[m][j].x, row_b[m][j].y, row_b[m][j].z, row_b[m][j].w};
                 const bool valid = tid + j * THREADS < (K >> 3);

@@ -29,14 +29,25 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
-// Round to nearest even; NaN stays a quiet NaN.
+// Round to nearest even; NaN stays a quiet NaN, (bits >> 16) | 0x0040.  gfx950 converts in hardware
+// (v_cvt_pk_bf16_f32); the instruction agrees with the integer formulation
+//   u += 0x7fff + ((u >> 16) & 1); return u >> 16     (NaN handled apart as above)
+// on every one of the 2^32 inputs.
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        return static_cast<uint16_t>((u >> 16) | 0x0040u);
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    const __bf16 b = static_cast<__bf16>(f);
+    uint16_t out;
+    __builtin_memcpy(&out, &b, 2);
+    return out;
+}
+
+// two conversions in one instruction: lo in bits 0..15, hi in bits 16..31
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t b = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
+    uint32_t out;
+    __builtin_memcpy(&out, &b, 4);
+    return out;
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {

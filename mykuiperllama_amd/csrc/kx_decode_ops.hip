@@ -25,10 +25,10 @@ __device__ __forceinline__ void unpack8(const uint4& raw, float (&out)[8]) {
 
 __device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
     uint4 out;
-    out.x = f32_to_bf16(v[0]) | (static_cast<uint32_t>(f32_to_bf16(v[1])) << 16);
-    out.y = f32_to_bf16(v[2]) | (static_cast<uint32_t>(f32_to_bf16(v[3])) << 16);
-    out.z = f32_to_bf16(v[4]) | (static_cast<uint32_t>(f32_to_bf16(v[5])) << 16);
-    out.w = f32_to_bf16(v[6]) | (static_cast<uint32_t>(f32_to_bf16(v[7])) << 16);
+    out.x = f32x2_to_bf16x2(v[0], v[1]);
+    out.y = f32x2_to_bf16x2(v[2], v[3]);
+    out.z = f32x2_to_bf16x2(v[4], v[5]);
+    out.w = f32x2_to_bf16x2(v[6], v[7]);
     return out;
 }
 
