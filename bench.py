@@ -137,7 +137,7 @@ def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager):
     model.set_input(1, ctx)  # every timed step decodes position `ctx` against ctx cached positions
     out = {"model": cfg_name, "context": ctx, "steps": steps, "launch": "eager" if eager else "hipGraph replay",
            "weights": "random-init INT4 AWQ group 128 (q/k/v and gate/up fused along N), bf16 embedding and lm_head",
-           "fusion": "add+RMSNorm and SwiGLU in the prologue of the consuming GEMV"}
+           "fusion": "add+RMSNorm and SwiGLU in the prologue of the consuming GEMV, QK-norm+RoPE+KV append in the epilogue of the q/k/v GEMV"}
     for with_head in (True, False):
         def launch(first, count, with_head=with_head):
             for _ in range(count):

@@ -113,6 +113,22 @@ int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t* delta, co
                              int32_t K, int32_t N, int32_t group_size, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* The front of a decoder layer in one launch (M = 1): add + RMSNorm as in kx_gemv_awq_addnorm_bf16,
+ * the fused q|k|v projection (N = (n_q_heads + 2 n_kv_heads) * 128, query heads first, then key
+ * heads, then value heads), and on the finished row what kx_qk_norm_rope_bf16 does: per-head RMSNorm
+ * of the query and key heads, rotation at *pos, queries to q_out, keys and values into row *pos of
+ * the caches.  Bitwise the result of kx_gemv_awq_addnorm_bf16 followed by kx_qk_norm_rope_bf16.
+ * n_q_heads + 2 n_kv_heads must be even (a column tile of 256 holds whole heads); head_dim = 128.
+ * Replaces: LayerAdd + LayerRMSNorm + LayerMatmul + LayerRMSNorm (heads) + LayerRope back to back
+ * (slots kuiper/include/op/layer.h:8-20; not implemented in the reference). */
+int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, const uint16_t* gain,
+                              float eps, uint16_t* residual_out, const int32_t* qweight,
+                              const uint16_t* scales, const int32_t* qzeros, const uint16_t* q_gain,
+                              const uint16_t* k_gain, uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache,
+                              int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
+                              float rope_theta, float qk_eps, int32_t K, int32_t group_size, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * BF16 GEMV fallback (non-quantised layers, lm_head):   y[m,n] = sum_k x[m,k] * W[n,k]
  *   W bf16 [N,K] row-major (dim0 = output features, dim1 = input features, the reading of

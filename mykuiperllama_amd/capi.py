@@ -26,6 +26,9 @@ SIGNATURES = {
     "kx_gemv_awq_swiglu_bf16": (ctypes.c_int, [_P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_addnorm_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I32, _I32,
                                                 _I32, _I32, _P, _SZ, _P]),
+    "kx_gemv_awq_qkv_rope_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _P, _P, _P, _P,
+                                                 _I32, _I32, _I32, _P, ctypes.c_float, ctypes.c_float, _I32, _I32,
+                                                 _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "kx_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
     "kx_add_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
@@ -128,6 +131,17 @@ def gemv_awq_addnorm_bf16(residual, delta, gain, eps, residual_out, qweight, sca
                                            _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y), M, K, N,
                                            group_size, _ptr(workspace),
                                            0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_awq_qkv_rope_bf16(residual, delta, gain, eps, residual_out, qweight, scales, qzeros, q_gain, k_gain,
+                           q_out, k_cache, v_cache, n_q, n_kv, pos, rope_theta, qk_eps, group_size, workspace):
+    """add + RMSNorm, fused q|k|v projection, per-head norm + rotation + cache append; one row."""
+    K = residual.shape[-1]
+    _check(load().kx_gemv_awq_qkv_rope_bf16(_ptr(residual), _ptr(delta), _ptr(gain), eps, _ptr(residual_out),
+                                            _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(q_gain), _ptr(k_gain),
+                                            _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n_q, n_kv, 128, _ptr(pos),
+                                            rope_theta, qk_eps, K, group_size, _ptr(workspace),
+                                            0 if workspace is None else workspace.numel(), _stream()))
 
 
 def set_awq_kernel_policy(policy):

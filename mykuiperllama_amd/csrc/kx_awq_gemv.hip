@@ -100,6 +100,18 @@ inline AwqPlan make_fused_plan(int M, int K, int N) {
     return p;
 }
 
+// One activation row, add + RMSNorm on the way in, per-head norm + rotation + cache append on the way out.
+template <int PRO>
+void launch_qkv(const AwqPlan& p, const FusedInput& fi, const RopeTarget& rope, const int32_t* qweight,
+                const uint16_t* scales, const int32_t* qzeros, float* partials, uint32_t* counters, int K, int N,
+                int group, hipStream_t stream) {
+#define KX_ARGS nullptr, qweight, scales, qzeros, nullptr, partials, counters, 1, K, N, group, p.coltiles, p.ktiles, 1, stream, fi, rope
+    if (p.waves == 8) launch_awq_gemv<8, 16, 1, PRO, kEpiQkRope>(KX_ARGS);
+    else if (p.rt == 16) launch_awq_gemv<4, 16, 1, PRO, kEpiQkRope>(KX_ARGS);
+    else launch_awq_gemv<4, 8, 1, PRO, kEpiQkRope>(KX_ARGS);
+#undef KX_ARGS
+}
+
 template <int PRO>
 void launch_fused(const AwqPlan& p, const FusedInput& fi, const int32_t* qweight, const uint16_t* scales,
                   const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters, int M, int K,
@@ -282,6 +294,53 @@ extern "C" int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t
     } else {
         kx::launch_fused<kx::kProAddNormLong>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N,
                                               group_size, kx::as_stream(stream));
+    }
+    return kx::launch_status();
+}
+
+extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, const uint16_t* gain,
+                                         float eps, uint16_t* residual_out, const int32_t* qweight,
+                                         const uint16_t* scales, const int32_t* qzeros, const uint16_t* q_gain,
+                                         const uint16_t* k_gain, uint16_t* q_out, uint16_t* k_cache,
+                                         uint16_t* v_cache, int32_t n_q_heads, int32_t n_kv_heads,
+                                         int32_t head_dim, const int32_t* pos, float rope_theta, float qk_eps,
+                                         int32_t K, int32_t group_size, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    if (!residual || !gain || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) {
+        return KX_ERR_NULL_POINTER;
+    }
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || !(rope_theta > 1.0f)) return KX_ERR_BAD_SHAPE;
+    // a column tile of 256 must hold whole heads
+    if ((n_q_heads + 2 * n_kv_heads) % (kx::kTileCols / kx::kHeadDim) != 0) return KX_ERR_BAD_SHAPE;
+    const int N = (n_q_heads + 2 * n_kv_heads) * kx::kHeadDim;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, q_out, 1, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    if (reinterpret_cast<uintptr_t>(residual) % 16 || reinterpret_cast<uintptr_t>(delta) % 16 ||
+        reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
+        return KX_ERR_ALIGNMENT;
+    }
+    if (residual_out == residual || (residual_out && residual_out == delta)) return KX_ERR_ALIAS;
+    const kx::AwqPlan p = kx::make_fused_plan(1, K, N);
+    if ((K >> 3) > kx::kNormChunks * p.waves * kx::kWave) return KX_ERR_BAD_SHAPE;
+    float* partials = nullptr;
+    uint32_t* counters = nullptr;
+    rc = kx::resolve_workspace(p, 1, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
+    kx::FusedInput fi{};
+    fi.a = residual;
+    fi.b = delta;
+    fi.gain = gain;
+    fi.r_out = residual_out;
+    fi.ld = K;
+    fi.eps = eps;
+    const kx::RopeTarget rope{q_gain, k_gain, q_out, k_cache, v_cache, pos, n_q_heads, n_kv_heads,
+                              log2f(rope_theta), qk_eps};
+    if ((K >> 3) <= p.waves * kx::kWave) {
+        kx::launch_qkv<kx::kProAddNorm>(p, fi, rope, qweight, scales, qzeros, partials, counters, K, N, group_size,
+                                        kx::as_stream(stream));
+    } else {
+        kx::launch_qkv<kx::kProAddNormLong>(p, fi, rope, qweight, scales, qzeros, partials, counters, K, N,
+                                            group_size, kx::as_stream(stream));
     }
     return kx::launch_status();
 }

@@ -21,6 +21,7 @@
 #define KX_AWQ_GEMV_KERNEL_H
 
 #include "kx_common.h"
+#include "kx_rope.h"
 #include "kx_splitk_exchange.h"
 
 namespace kx {
@@ -99,12 +100,16 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(va, vb, c, false);
 }
 
-template <int WAVES, int RT, int MB, int PRO>
+// What happens to the finished sums (EPI below).
+constexpr int kEpiStore = 0;   // y[m, n] = bf16(sum)
+constexpr int kEpiQkRope = 1;  // the row is q | k | v heads of 128: per-head norm, rotation, cache append (M = 1)
+
+template <int WAVES, int RT, int MB, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi) {
+    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi, RopeTarget rope) {
     constexpr int SLOTS = WAVES * kSlotsPerWave;
     constexpr int KB = SLOTS * RT;
     constexpr int THREADS = WAVES * kWave;
@@ -352,21 +357,42 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     }
 
     __shared__ uint32_t s_prev;
-    splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
-                              &s_prev);
+    if constexpr (EPI == kEpiStore) {
+        splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
+                                  &s_prev);
+    } else {
+        static_assert(MB == 1, "the rotary epilogue serves one activation row");
+        float sum[MB];
+        if (!splitk_exchange_sum<MB>(psum, sum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials,
+                                     counters, &s_prev)) {
+            return;
+        }
+        // A column tile is two heads of 128.  The finished row, rounded to bf16 as a separate GEMV
+        // would store it, goes through LDS so that the first wave of each head holds elements i and
+        // i + 64 in lane i, the layout of the per-head routine.
+        __shared__ uint16_t s_row[kTileCols];
+        if (tid < kTileCols) s_row[tid] = f32_to_bf16(sum[0]);
+        __syncthreads();
+        if (tid < kTileCols && (tid & 64) == 0) {
+            const int local = tid >> 7;
+            const int head = ct * (kTileCols / kHeadDim) + local;
+            qk_norm_rope_head(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane, rope);
+        }
+    }
 }
 
-template <int WAVES, int RT, int MB, int PRO = kProNone>
+template <int WAVES, int RT, int MB, int PRO = kProNone, int EPI = kEpiStore>
 inline void launch_awq_gemv(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
                             const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
                             int M, int K, int N, int group, int coltiles, int ktiles, int mtiles,
-                            hipStream_t stream, const FusedInput& fi = FusedInput{}) {
+                            hipStream_t stream, const FusedInput& fi = FusedInput{},
+                            const RopeTarget& rope = RopeTarget{}) {
     dim3 grid(coltiles * ktiles, mtiles, 1);
     dim3 block(WAVES * kWave, 1, 1);
-    hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB, PRO>), grid, block, 0, stream, x,
+    hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB, PRO, EPI>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group, coltiles, ktiles, fi);
+                       group, coltiles, ktiles, fi, rope);
 }
 
 }  // namespace kx

@@ -8,6 +8,7 @@
 // buffers (model::ModelBufferType, kuiper/include/base/base.h:12-31) but implements none of them
 // except the fp32 add (kuiper/source/op/kernel/cuda/add_kernel.cu:4-12).
 #include "kx_common.h"
+#include "kx_rope.h"
 
 #include <math.h>
 
@@ -107,47 +108,12 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(uint16_t* __restr
 //   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
 //   out[i + 64] = x[i+64] * cos(pos f_i) + x[i] * sin(pos f_i),     f_i = theta^(-i/64)
 // ------------------------------------------------------------------------------------------------
-constexpr int kHeadDim = 128;
-
-__global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __restrict__ qkv,
-                                                           const uint16_t* __restrict__ q_gain,
-                                                           const uint16_t* __restrict__ k_gain,
-                                                           uint16_t* __restrict__ q_out,
-                                                           uint16_t* __restrict__ k_cache,
-                                                           uint16_t* __restrict__ v_cache, int n_q, int n_kv,
-                                                           const int32_t* __restrict__ pos_ptr, float log2_theta,
-                                                           float eps) {
+__global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __restrict__ qkv, RopeTarget t) {
     const int head = blockIdx.x * 4 + threadIdx.x / kWave;  // 0 .. n_q + 2 n_kv - 1
     const int lane = threadIdx.x % kWave;
-    if (head >= n_q + 2 * n_kv) return;
-    const int pos = pos_ptr[0];
+    if (head >= t.n_q + 2 * t.n_kv) return;
     const uint16_t* src = qkv + static_cast<size_t>(head) * kHeadDim;
-    const float a = bf16_to_f32(src[lane]);
-    const float b = bf16_to_f32(src[lane + 64]);
-    if (head >= n_q + n_kv) {  // value head: straight into the cache
-        uint16_t* dst = v_cache + (static_cast<size_t>(pos) * n_kv + (head - n_q - n_kv)) * kHeadDim;
-        dst[lane] = src[lane];
-        dst[lane + 64] = src[lane + 64];
-        return;
-    }
-    const bool is_q = head < n_q;
-    const uint16_t* gain = is_q ? q_gain : k_gain;
-    const float ss = wave_sum(a * a + b * b);
-    const float inv = 1.0f / sqrtf(ss / static_cast<float>(kHeadDim) + eps);
-    const float na = bf16_to_f32(gain[lane]) * bf16_to_f32(f32_to_bf16(a * inv));
-    const float nb = bf16_to_f32(gain[lane + 64]) * bf16_to_f32(f32_to_bf16(b * inv));
-    // the norm output is a bf16 tensor in the usual formulation; the rotation starts from that
-    const float xa = bf16_to_f32(f32_to_bf16(na));
-    const float xb = bf16_to_f32(f32_to_bf16(nb));
-    const float freq = exp2f(-log2_theta * static_cast<float>(lane) / 64.0f);
-    float s, c;
-    sincosf(static_cast<float>(pos) * freq, &s, &c);
-    const float oa = xa * c - xb * s;
-    const float ob = xb * c + xa * s;
-    uint16_t* dst = is_q ? q_out + static_cast<size_t>(head) * kHeadDim
-                         : k_cache + (static_cast<size_t>(pos) * n_kv + (head - n_q)) * kHeadDim;
-    dst[lane] = f32_to_bf16(oa);
-    dst[lane + 64] = f32_to_bf16(ob);
+    qk_norm_rope_head(src[lane], src[lane + 64], head, lane, t);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -533,8 +499,8 @@ extern "C" int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain,
     if (!qkv || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) return KX_ERR_NULL_POINTER;
     if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || !(rope_theta > 1.0f)) return KX_ERR_BAD_SHAPE;
     const int heads = n_q_heads + 2 * n_kv_heads;
-    hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4), dim3(256), 0, kx::as_stream(stream), qkv,
-                       q_gain, k_gain, q_out, k_cache, v_cache, n_q_heads, n_kv_heads, pos, log2f(rope_theta), eps);
+    kx::RopeTarget t{q_gain, k_gain, q_out, k_cache, v_cache, pos, n_q_heads, n_kv_heads, log2f(rope_theta), eps};
+    hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4), dim3(256), 0, kx::as_stream(stream), qkv, t);
     return kx::launch_status();
 }
 

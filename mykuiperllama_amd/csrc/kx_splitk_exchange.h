@@ -28,23 +28,20 @@ __device__ __forceinline__ float load_agent(const float* p) {
 
 // Called by every thread of the workgroup (it contains barriers).  Thread tid < 256 owns tile column
 // tid and brings psum[r], its partial sum for activation row m0 + r.  `s_prev` is one uint32 of LDS.
+// Returns true, the same in every thread, in the workgroup that ends up with the finished sums
+// (in `sum`, for the threads that own a column); the others return false and are done.
 template <int ROWS>
-__device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS], int m0, int M, int N,
-                                                      int ct, int kt, int ktiles, int counter_index,
-                                                      float* __restrict__ partials,
-                                                      uint32_t* __restrict__ counters,
-                                                      uint16_t* __restrict__ y, uint32_t* s_prev) {
+__device__ __forceinline__ bool splitk_exchange_sum(const float (&psum)[ROWS], float (&sum)[ROWS], int m0, int M,
+                                                    int N, int ct, int kt, int ktiles, int counter_index,
+                                                    float* __restrict__ partials,
+                                                    uint32_t* __restrict__ counters, uint32_t* s_prev) {
     const int tid = threadIdx.x;
     const int col = ct * kTileCols + tid;
     const bool col_ok = (tid < kTileCols) && (col < N);
     if (ktiles == 1) {
-        if (col_ok) {
 #pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(psum[r]);
-            }
-        }
-        return;
+        for (int r = 0; r < ROWS; r++) sum[r] = psum[r];
+        return true;
     }
 
     const size_t tstride = static_cast<size_t>(M) * N;  // floats between consecutive K tiles
@@ -64,16 +61,15 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
         *s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return;
+    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return false;
 
     // Last to arrive: every other workgroup's partials were acknowledged before its increment.
     // Up to 64 loads are in flight per thread (TB K-tiles of every row at a time); per row the
     // additions keep the order t = 0, 1, 2, ...
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) sum[r] = 0.0f;
     if (col_ok) {
         constexpr int TB = ROWS >= 16 ? 4 : 16;
-        float sum[ROWS];
-#pragma unroll
-        for (int r = 0; r < ROWS; r++) sum[r] = 0.0f;
         const float* pp = partials + col;
         for (int t0 = 0; t0 < ktiles; t0 += TB) {
             float v[ROWS][TB];
@@ -92,14 +88,31 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
                 for (int u = 0; u < TB; u++) sum[r] += v[r][u];
             }
         }
-#pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(sum[r]);
-        }
     }
     if (tid == 0) {
         // leave the workspace ready for the next launch
         __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+
+// The exchange followed by the plain epilogue: y[m, col] = bf16(sum).
+template <int ROWS>
+__device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS], int m0, int M, int N,
+                                                      int ct, int kt, int ktiles, int counter_index,
+                                                      float* __restrict__ partials,
+                                                      uint32_t* __restrict__ counters,
+                                                      uint16_t* __restrict__ y, uint32_t* s_prev) {
+    float sum[ROWS];
+    if (!splitk_exchange_sum<ROWS>(psum, sum, m0, M, N, ct, kt, ktiles, counter_index, partials, counters, s_prev)) {
+        return;
+    }
+    const int col = ct * kTileCols + static_cast<int>(threadIdx.x);
+    if (threadIdx.x < kTileCols && col < N) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(sum[r]);
+        }
     }
 }
 

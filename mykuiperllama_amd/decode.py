@@ -14,8 +14,9 @@ q/k/v share one fused GEMV (N = (n_q + 2 n_kv) * 128) and gate/up another (N = 2
 packed tensors of the separate projections are concatenated along N when the weights are loaded
 (rows are laid end to end; the nibble order inside a word is untouched).  The residual add is fused
 into the next RMSNorm, and by default (`fused=True`) both ride in the prologue of the GEMV that
-consumes the normalised row, as does SwiGLU in front of the down projection: seven launches per
-layer instead of ten.  The residual stream then alternates between two buffers, because a fused
+consumes the normalised row, as does SwiGLU in front of the down projection, and the per-head
+norm, rotation and cache append ride in the epilogue of the q/k/v GEMV: six launches per layer
+instead of ten.  The residual stream then alternates between two buffers, because a fused
 launch reads the whole incoming row in every workgroup while it writes the updated one.
 Every launch goes to torch's current stream, so a step can be captured in a HIP graph; token and
 position live in device memory for that reason.
@@ -167,10 +168,9 @@ class DecodeModel:
         xa, xb = self.x, self.x2
         for li, L in enumerate(self.layers):
             qw, sc, qz = L["qkv"]
-            capi.gemv_awq_addnorm_bf16(xa, None if li == 0 else self.down, L["in_norm"], c.eps, xb, qw, sc, qz,
-                                       self.qkv, g, ws)
-            capi.qk_norm_rope_bf16(self.qkv, L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
-                                   c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps)
+            capi.gemv_awq_qkv_rope_bf16(xa, None if li == 0 else self.down, L["in_norm"], c.eps, xb, qw, sc, qz,
+                                        L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
+                                        c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps, g, ws)
             capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
                                   self.max_positions, self.attn_ws)
             self._awq(self.attn, L["o"], self.o)
@@ -185,7 +185,7 @@ class DecodeModel:
             capi.argmax_bf16(self.logits, self.next_token)
 
     def launches_per_step(self, with_lm_head=True, fused=True):
-        return 1 + self.cfg.layers * (7 if fused else 10) + 1 + (2 if with_lm_head else 0)
+        return 1 + self.cfg.layers * (6 if fused else 10) + 1 + (2 if with_lm_head else 0)
 
 
 def step_bytes(cfg, ctx, with_lm_head=True):

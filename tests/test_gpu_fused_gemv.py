@@ -156,6 +156,83 @@ def test_addnorm_prologue_equals_separate_launches(capi, torch, oracle, M, K, N,
     oracle_check(oracle, torch, p, h_sep, y_fused)
 
 
+QKV_CASES = [
+    # hidden K, n_q, n_kv, group, with delta
+    (4096, 32, 8, 128, True),    # Qwen3-8B
+    (5120, 64, 8, 128, True),    # Qwen3-32B
+    (4096, 32, 8, 128, False),   # first layer: no delta
+    (512, 4, 2, 128, True),
+    (128, 2, 1, 32, True),       # four waves per workgroup
+    (64, 2, 2, 32, True),        # K in one workgroup: no split, every workgroup finishes its own tile
+]
+
+
+@pytest.mark.parametrize("K,n_q,n_kv,group,with_delta", QKV_CASES)
+def test_qkv_rope_launch_equals_separate_launches(capi, torch, K, n_q, n_kv, group, with_delta):
+    eps, theta, pos_value, max_pos = 1e-6, 1e6, 37, 48
+    N = (n_q + 2 * n_kv) * 128
+    _, (qw, sc, qz) = weights(torch, f"fused_qkv_{K}_{n_q}_{n_kv}", 1, K, N, group)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(K + n_q)
+    resid = (torch.randn((1, K), device="cuda", generator=g) * 2.0).bfloat16()
+    delta = torch.randn((1, K), device="cuda", generator=g).bfloat16() if with_delta else None
+    gain = (1 + 0.1 * torch.randn((K,), device="cuda", generator=g)).bfloat16()
+    q_gain = (1 + 0.1 * torch.randn((128,), device="cuda", generator=g)).bfloat16()
+    k_gain = (1 + 0.1 * torch.randn((128,), device="cuda", generator=g)).bfloat16()
+    pos = torch.tensor([pos_value], dtype=torch.int32, device="cuda")
+    ws = capi.make_workspace(1, K, N)
+
+    def caches():
+        return (torch.full((max_pos, n_kv, 128), 3.0, dtype=torch.bfloat16, device="cuda"),
+                torch.full((max_pos, n_kv, 128), 5.0, dtype=torch.bfloat16, device="cuda"))
+
+    # separate: add + norm + GEMV, then the stand-alone per-head kernel
+    k_sep, v_sep = caches()
+    qkv = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
+    r_sep = torch.empty((1, K), dtype=torch.bfloat16, device="cuda")
+    q_sep = torch.empty((1, n_q * 128), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_addnorm_bf16(resid, delta, gain, eps, r_sep, qw, sc, qz, qkv, group, ws)
+    capi.qk_norm_rope_bf16(qkv, q_gain, k_gain, q_sep, k_sep, v_sep, n_q, n_kv, pos, theta, eps)
+    # one launch
+    k_one, v_one = caches()
+    r_one = torch.empty((1, K), dtype=torch.bfloat16, device="cuda")
+    q_one = torch.full((1, n_q * 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_qkv_rope_bf16(resid, delta, gain, eps, r_one, qw, sc, qz, q_gain, k_gain, q_one, k_one, v_one,
+                                n_q, n_kv, pos, theta, eps, group, ws)
+    torch.cuda.synchronize()
+    for a, b in ((q_one, q_sep), (k_one, k_sep), (v_one, v_sep), (r_one, r_sep)):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # only row `pos` of the caches was touched
+    assert (k_one[:pos_value] == 3.0).all() and (k_one[pos_value + 1:] == 3.0).all()
+    assert (v_one[:pos_value] == 5.0).all() and (v_one[pos_value + 1:] == 5.0).all()
+    assert torch.isfinite(q_one.float()).all()
+
+
+def test_qkv_rope_launch_rejects_bad_arguments(capi, torch):
+    K, n_q, n_kv, group = 256, 3, 1, 128  # five heads do not fill column tiles of two heads
+    N = (n_q + 2 * n_kv) * 128
+    _, (qw, sc, qz) = weights(torch, "fused_qkv_bad", 1, K, N, group)
+    x = torch.zeros((1, K), dtype=torch.bfloat16, device="cuda")
+    gain = torch.ones((K,), dtype=torch.bfloat16, device="cuda")
+    hg = torch.ones((128,), dtype=torch.bfloat16, device="cuda")
+    q = torch.zeros((1, n_q * 128), dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros((4, n_kv, 128), dtype=torch.bfloat16, device="cuda")
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ws = capi.make_workspace(1, K, N)
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_qkv_rope_bf16(x, None, gain, 1e-6, None, qw, sc, qz, hg, hg, q, kc, kc.clone(), n_q, n_kv, pos,
+                                    1e6, 1e-6, group, ws)
+    assert e.value.code == -2
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_qkv_rope_bf16(x, None, gain, 1e-6, x, qw, sc, qz, hg, hg, q, kc, kc.clone(), 2, 1, pos,
+                                    1e6, 1e-6, group, ws)
+    assert e.value.code == -5
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_qkv_rope_bf16(x, None, gain, 1e-6, None, qw, sc, qz, hg, hg, q, kc, kc.clone(), 2, 1, None,
+                                    1e6, 1e-6, group, ws)
+    assert e.value.code == -1
+
+
 def test_fused_launches_are_deterministic_and_leave_the_workspace_reusable(capi, torch):
     M, K, N, group = 1, 4096, 6144, 128
     _, (qw, sc, qz) = weights(torch, "fused_repeat", M, K, N, group)
