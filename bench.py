@@ -14,6 +14,9 @@ Prints one JSON line:  value = algorithmic bytes of a step / time of a step, in 
   cpu_baseline  the oracle's single-threaded fp32 restatement, timed on this host on a bounded
                 number of passes over the same seven shapes
   per_shape     each projection shape on its own, cold weights, same event timing
+  small_batch   configs[2]: M in {1, 2, 4, 8, 16} on three shapes, microseconds per launch of the
+                vector-ALU kernel and of the MFMA kernel (cold weights, same event timing)
+  decode        configs[3] (and configs[4] with --decode-32b): tokens/s of a full decode step
 """
 import argparse
 import json
@@ -31,7 +34,7 @@ METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
 # HBM bytes per launch of the dominant kernel (average over the seven launches of a step) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
 # reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).
-TRAFFIC_BYTES_PER_LAUNCH = 15374000
+TRAFFIC_BYTES_PER_LAUNCH = 15370600
 
 
 def parse_args():
@@ -43,6 +46,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-passes", type=int, default=30)
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--no-small-batch", action="store_true", help="skip the M = 1..16 vector/MFMA kernel table")
     ap.add_argument("--no-decode", action="store_true", help="skip the Qwen3-8B decode-step measurement")
     ap.add_argument("--decode-32b", action="store_true", help="also run the Qwen3-32B-shaped decode step")
     ap.add_argument("--decode-steps", type=int, default=60)
@@ -226,6 +230,55 @@ def main():
                                          "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
                                          "bytes": b}
 
+        # the two launches a decode step fuses along N, same cold-weight protocol
+        fused_shapes = {"qkv fused": (4096, 6144), "gate+up fused": (4096, 24576)}
+        fsets = [WeightSet(torch, fused_shapes, group, gen) for _ in range(WEIGHT_SETS)]
+        for n, (K, N) in fused_shapes.items():
+            b = synth.awq_gemv_bytes(1, K, N)
+            yf = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
+            wsf = capi.make_workspace(1, K, N)
+            reps = 240 // WEIGHT_SETS * WEIGHT_SETS
+
+            def launch_f(first, count, n=n, yf=yf, wsf=wsf, K=K):
+                for s in range(first, first + count):
+                    qw, sc, qz = fsets[s % WEIGHT_SETS].t[n]
+                    capi.gemv_awq_bf16(xs[K], qw, sc, qz, yf, group, wsf)
+
+            sec = timed_region(torch, launch_f, reps, WEIGHT_SETS, args.eager, WEIGHT_SETS)
+            us = sec / reps * 1e6
+            per_shape[f"{n} {K}x{N}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
+                                         "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                                         "bytes": b}
+        del fsets
+        torch.cuda.empty_cache()
+
+    small_batch = None
+    if not args.no_small_batch:
+        small_batch = {"unit": "us per launch", "kernels": {"vector": "VALU kernel, bf16 dot2", "mfma": "16x16x32 bf16 MFMA"}}
+        for n in ["q_proj", "gate_proj", "down_proj"]:
+            K, N = shapes[n]
+            row = {}
+            for M in (1, 2, 4, 8, 16):
+                xm = torch.randn((M, K), device="cuda", generator=gen).bfloat16()
+                ym = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+                wsm = capi.make_workspace(M, K, N)
+                cell = {}
+                for label, policy in (("vector", 1), ("mfma", 2)):
+                    capi.set_awq_kernel_policy(policy)
+
+                    def launch_m(first, count, n=n, xm=xm, ym=ym, wsm=wsm):
+                        for s in range(first, first + count):
+                            qw, sc, qz = sets[s % WEIGHT_SETS].t[n]
+                            capi.gemv_awq_bf16(xm, qw, sc, qz, ym, group, wsm)
+
+                    reps = 10 * WEIGHT_SETS
+                    sec = timed_region(torch, launch_m, reps, WEIGHT_SETS, args.eager, WEIGHT_SETS)
+                    cell[label] = round(sec / reps * 1e6, 2)
+                capi.set_awq_kernel_policy(0)
+                cell["GB/s_best"] = round(synth.awq_gemv_bytes(M, K, N) / min(cell["vector"], cell["mfma"]) / 1e3, 1)
+                row[f"M={M}"] = cell
+            small_batch[f"{n} {K}x{N}"] = row
+
     out = {
         "metric": METRIC,
         "value": round(value, 2),
@@ -252,6 +305,8 @@ def main():
     }
     if per_shape is not None:
         out["per_shape"] = per_shape
+    if small_batch is not None:
+        out["small_batch"] = small_batch
     if not args.no_decode:
         del sets
         torch.cuda.empty_cache()
