@@ -3,6 +3,7 @@
   libkx_hip.so   HIP kernels + C ABI            (csrc/*.hip)
   libkuiper.so   C++ host API over that C ABI    (kuiper/source/**/*.cpp)
   test_kuiper    C++ test runner for the host API (tests/cpp/*, links oracle/kx_oracle.c)
+  kx_safetensors_dump   lists the tensors of a checkpoint file (kuiper/app/safetensors_dump.cpp)
 
 Everything lands under mykuiperllama_amd/lib/, in-tree, so that a snapshot of the repository
 carries the binaries to a machine that only runs them.
@@ -22,6 +23,7 @@ TESTS_CPP = os.path.join(ROOT, "tests", "cpp")
 KX_LIB = os.path.join(LIB_DIR, "libkx_hip.so")
 KUIPER_LIB = os.path.join(LIB_DIR, "libkuiper.so")
 KUIPER_TEST = os.path.join(LIB_DIR, "test_kuiper")
+SAFETENSORS_DUMP = os.path.join(LIB_DIR, "kx_safetensors_dump")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU forms are switched off for all device code
@@ -53,6 +55,8 @@ def build_kuiper():
     inc = ["-I", INCLUDE, "-I", os.path.join(KUIPER, "include"), "-I", os.path.join(KUIPER, "source", "op")]
     _run([HIPCC] + DEVICE_FLAGS + COMMON + ["-shared"] + inc + srcs +
          ["-L", LIB_DIR, "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", KUIPER_LIB])
+    _run([HIPCC, "--offload-arch=gfx950"] + COMMON + inc + [os.path.join(KUIPER, "app", "safetensors_dump.cpp")] +
+         ["-L", LIB_DIR, "-lkuiper", "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", SAFETENSORS_DUMP])
     # C++ tests of the host API live under tests/cpp and link the CPU oracle as their checker
     tests = sorted(glob.glob(os.path.join(TESTS_CPP, "*.cpp")) + glob.glob(os.path.join(TESTS_CPP, "*.hip")))
     if tests:

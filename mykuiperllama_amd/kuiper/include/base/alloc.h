@@ -42,11 +42,37 @@ public:
     void release(void* ptr) const override;
 };
 
+// GPU memory with a free-block pool.  release() keeps the block; allocate() takes the smallest idle
+// block that fits without wasting more than half of it, else calls hipMalloc.  hipMalloc and
+// hipFree cost tens of microseconds to milliseconds and hipFree waits for the device, which a
+// decode loop that creates tensors per step cannot afford; the reference does one cudaMalloc and
+// one cudaFree per buffer (kuiper/source/base/alloc_cu.cpp:8-23).  Blocks are handed out again in
+// program order, so work that still uses a released block must be on the stream that the next
+// user launches on, or finished (the rule of any caching allocator).
 class CUDADeviceAllocator : public DeviceAllocator {
 public:
+    struct PoolStats {
+        size_t device_allocations = 0;  // hipMalloc calls
+        size_t device_frees = 0;        // hipFree calls
+        size_t reuses = 0;              // allocate() calls served from the pool
+        size_t idle_bytes = 0;          // bytes held in idle blocks
+        size_t busy_bytes = 0;          // bytes handed out
+    };
+
     explicit CUDADeviceAllocator();
+    ~CUDADeviceAllocator() override;
     void* allocate(size_t byte_size) const override;
     void release(void* ptr) const override;
+
+    // Idle blocks beyond this many bytes are returned to the device, largest first (default 1 GiB;
+    // 0 switches pooling off: every release is a hipFree, as in the reference).
+    void set_idle_limit(size_t bytes);
+    void trim();  // returns every idle block to the device
+    PoolStats stats() const;
+
+private:
+    struct Pool;
+    std::unique_ptr<Pool> pool_;
 };
 
 // One shared allocator per kind, created on first use (not synchronised: the host API is
