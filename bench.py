@@ -44,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--eager", action="store_true", help="launch from the host loop instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-passes", type=int, default=30)
+    ap.add_argument("--cpu-passes", type=int, default=150)
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-small-batch", action="store_true", help="skip the M = 1..16 vector/MFMA kernel table")
     ap.add_argument("--no-decode", action="store_true", help="skip the Qwen3-8B decode-step measurement")
