@@ -125,11 +125,24 @@ def cpu_baseline(passes):
             oracle.gemv_awq_f32(p["x"], p["qweight"], p["scales"], p["qzeros"], p["group"])
     dt = time.perf_counter() - t0
     del np
-    return {"value": round(step_bytes * passes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "ms_per_step": round(dt / passes * 1e3, 2),
-            "sample": f"{passes} passes over the seven Qwen3-8B projections at M=1 (seeded inputs), "
-                      f"oracle/kx_oracle.c kxo_gemv_awq_f32, gcc -O3 -march=x86-64-v3, one thread, "
-                      f"host has {os.cpu_count()} logical cpus"}
+    out = {"value": round(step_bytes * passes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+           "ms_per_step": round(dt / passes * 1e3, 2),
+           "sample": f"{passes} passes over the seven Qwen3-8B projections at M=1 (seeded inputs), "
+                     f"oracle/kx_oracle.c kxo_gemv_awq_f32, gcc -O3 -march=x86-64-v3, one thread, "
+                     f"host has {os.cpu_count()} logical cpus"}
+    # the same arithmetic spread over the host's cores (columns split across threads), as a second figure
+    threads = min(os.cpu_count() or 1, 16)
+    if threads > 1:
+        mt_passes = max(10, passes // 3)
+        t0 = time.perf_counter()
+        for _ in range(mt_passes):
+            for p in probs:
+                oracle.gemv_awq_f32_threads(p["x"], p["qweight"], p["scales"], p["qzeros"], p["group"], threads)
+        dt = time.perf_counter() - t0
+        out["all_cores"] = {"value": round(step_bytes * mt_passes / dt / 1e9, 4), "unit": "GB/s", "cores": threads,
+                            "ms_per_step": round(dt / mt_passes * 1e3, 2),
+                            "sample": f"{mt_passes} passes, kxo_gemv_awq_f32_range over {threads} threads"}
+    return out
 
 
 def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager):

@@ -213,12 +213,15 @@ int kxo_gemv_awq_f64(const uint16_t* x_bf16, const int32_t* qweight, const uint1
     return 0;
 }
 
-int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint16_t* scales_f16,
-                     const int32_t* qzeros, int64_t M, int64_t K, int64_t N, int64_t group,
-                     uint16_t* y_bf16) {
+/* word columns [j_begin, j_end) of the fp32 evaluation; the arithmetic of a column does not depend
+ * on the range it is computed in */
+int kxo_gemv_awq_f32_range(const uint16_t* x_bf16, const int32_t* qweight, const uint16_t* scales_f16,
+                           const int32_t* qzeros, int64_t M, int64_t K, int64_t N, int64_t group,
+                           int64_t j_begin, int64_t j_end, uint16_t* y_bf16) {
     if (group <= 0 || (K % group) != 0 || (N % 8) != 0) return 1;
     int64_t wcols = N / 8;
     int64_t groups = K / group;
+    if (j_begin < 0 || j_end > wcols || j_begin > j_end) return 1;
     float* acc = (float*)malloc((size_t)N * sizeof(float));
     float* sg = (float*)malloc((size_t)N * sizeof(float));
     float* zg = (float*)malloc((size_t)N * sizeof(float));
@@ -229,10 +232,10 @@ int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint1
         return 3;
     }
     for (int64_t m = 0; m < M; m++) {
-        for (int64_t n = 0; n < N; n++) acc[n] = 0.0f;
+        for (int64_t n = 8 * j_begin; n < 8 * j_end; n++) acc[n] = 0.0f;
         for (int64_t g = 0; g < groups; g++) {
             /* per-group scales and zero points, unpacked once */
-            for (int64_t j = 0; j < wcols; j++) {
+            for (int64_t j = j_begin; j < j_end; j++) {
                 uint32_t zw = (uint32_t)qzeros[g * wcols + j];
                 for (int i = 0; i < 8; i++) {
                     int64_t n = 8 * j + KXO_ORDER[i];
@@ -243,7 +246,7 @@ int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint1
             for (int64_t k = g * group; k < (g + 1) * group; k++) {
                 float xv = kxo_bf16_to_f32(x_bf16[m * K + k]);
                 const int32_t* row = qweight + k * wcols;
-                for (int64_t j = 0; j < wcols; j++) {
+                for (int64_t j = j_begin; j < j_end; j++) {
                     uint32_t qw = (uint32_t)row[j];
                     for (int i = 0; i < 8; i++) {
                         int64_t n = 8 * j + KXO_ORDER[i];
@@ -253,12 +256,19 @@ int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint1
                 }
             }
         }
-        for (int64_t n = 0; n < N; n++) y_bf16[m * N + n] = kxo_f32_to_bf16(acc[n]);
+        for (int64_t n = 8 * j_begin; n < 8 * j_end; n++) y_bf16[m * N + n] = kxo_f32_to_bf16(acc[n]);
     }
     free(acc);
     free(sg);
     free(zg);
     return 0;
+}
+
+int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint16_t* scales_f16,
+                     const int32_t* qzeros, int64_t M, int64_t K, int64_t N, int64_t group,
+                     uint16_t* y_bf16) {
+    if ((N % 8) != 0) return 1;
+    return kxo_gemv_awq_f32_range(x_bf16, qweight, scales_f16, qzeros, M, K, N, group, 0, N / 8, y_bf16);
 }
 
 /* ------------------------------------------------------------------ BF16 GEMV */

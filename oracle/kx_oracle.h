@@ -74,6 +74,13 @@ int kxo_gemv_awq_f32(const uint16_t* x_bf16, const int32_t* qweight, const uint1
                      const int32_t* qzeros, int64_t M, int64_t K, int64_t N, int64_t group,
                      uint16_t* y_bf16);
 
+/* The same for the word columns [j_begin, j_end) only (columns 8*j_begin .. 8*j_end-1 of y are
+ * written): lets a caller spread one GEMV over threads.  Pinned by the full-range function, of
+ * which it is the body: any split returns the same bits. */
+int kxo_gemv_awq_f32_range(const uint16_t* x_bf16, const int32_t* qweight, const uint16_t* scales_f16,
+                           const int32_t* qzeros, int64_t M, int64_t K, int64_t N, int64_t group,
+                           int64_t j_begin, int64_t j_end, uint16_t* y_bf16);
+
 /* ---- BF16 GEMV: y[m,n] = sum_k x[m,k] * W[n,k], W bf16 row-major [N, K] ---- */
 int kxo_gemv_bf16_f64(const uint16_t* x_bf16, const uint16_t* w_bf16, int64_t M, int64_t K,
                       int64_t N, double* y_f64);

@@ -55,6 +55,8 @@ def _declare(L):
     L.kxo_awq_dequant_one.restype = ctypes.c_uint16
     L.kxo_gemv_awq_f64.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
     L.kxo_gemv_awq_f32.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
+    L.kxo_gemv_awq_f32_range.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+    L.kxo_gemv_awq_f32_range.restype = ctypes.c_int
     L.kxo_gemv_bf16_f64.argtypes = [_P, _P, _I, _I, _I, _P]
     L.kxo_gemv_bf16_f32.argtypes = [_P, _P, _I, _I, _I, _P]
     for f in (L.kxo_awq_pack, L.kxo_awq_unpack, L.kxo_awq_dequant_bf16, L.kxo_gemv_awq_f64,
@@ -172,6 +174,27 @@ def gemv_awq_f32(x_bf16, qweight, scales_f16, qzeros, group):
     y = np.empty((M, N), np.uint16)
     _check(lib().kxo_gemv_awq_f32(_ptr(x_bf16), _ptr(qweight), _ptr(scales_f16), _ptr(qzeros),
                                   M, K, N, group, _ptr(y)), "gemv_awq_f32")
+    return y
+
+
+def gemv_awq_f32_threads(x_bf16, qweight, scales_f16, qzeros, group, threads):
+    """The fp32 evaluation spread over `threads` host threads, each a contiguous range of word columns
+    (the C call releases the interpreter lock).  Same bits as gemv_awq_f32 for any thread count."""
+    from concurrent.futures import ThreadPoolExecutor
+    x_bf16, qweight, scales_f16, qzeros, M, K, N = _awq_args(x_bf16, qweight, scales_f16, qzeros,
+                                                             group)
+    y = np.empty((M, N), np.uint16)
+    wcols = N // 8
+    threads = max(1, min(threads, wcols))
+    bounds = [wcols * t // threads for t in range(threads + 1)]
+
+    def work(t):
+        return lib().kxo_gemv_awq_f32_range(_ptr(x_bf16), _ptr(qweight), _ptr(scales_f16), _ptr(qzeros),
+                                            M, K, N, group, bounds[t], bounds[t + 1], _ptr(y))
+
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        for rc in pool.map(work, range(threads)):
+            _check(rc, "gemv_awq_f32_range")
     return y
 
 

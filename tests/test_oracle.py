@@ -258,3 +258,13 @@ def test_bf16_gemv_matches_torch(oracle, M, K, N):
     x1 = np.zeros((1, K), np.uint16)
     x1[0, 5] = 0x3F80
     assert np.array_equal(oracle.gemv_bf16_f32(x1, p["w"])[0], p["w"][:, 5])
+
+
+def test_threaded_fp32_gemv_returns_the_single_thread_bits(oracle):
+    """The column-range entry point is the body of the full-range one: any split gives the same bits."""
+    from mykuiperllama_amd import synth
+    p = synth.make_awq_problem("threads", 2, 512, 1064, 128)
+    one = oracle.gemv_awq_f32(p["x"], p["qweight"], p["scales"], p["qzeros"], p["group"])
+    for threads in (1, 2, 3, 7, 133, 1000):
+        many = oracle.gemv_awq_f32_threads(p["x"], p["qweight"], p["scales"], p["qzeros"], p["group"], threads)
+        assert np.array_equal(one, many), threads
