@@ -67,7 +67,12 @@ def kernel_policy(request, capi):
     capi.set_awq_kernel_policy(0)
 
 
-@pytest.mark.parametrize("K,N", [(1024, 2048)] + SHAPES_8B)
+SHAPES_32B = sorted(set(synth.QWEN3_32B.values()))
+# the launches a decode step fuses along N; 4096 -> 24576 takes the 32-rows-per-lane plan
+SHAPES_FUSED = [(4096, 6144), (4096, 24576), (5120, 10240)]
+
+
+@pytest.mark.parametrize("K,N", [(1024, 2048)] + SHAPES_8B + SHAPES_32B + SHAPES_FUSED)
 def test_gemv_m1_matches_oracle(capi, torch, oracle, K, N):
     p = synth.make_awq_problem(f"gemv_m1_{K}x{N}", 1, K, N)
     y, _ = run_awq(capi, torch, p)
