@@ -169,9 +169,11 @@ int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const in
  *                         (bf16 [max_positions][n_kv_heads][128]).  head_dim must be 128.
  *   kx_attn_decode_bf16   GQA attention of one query position against cache rows 0 .. *pos:
  *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv in
- *                         {1,2,4,8}; split over the context in chunks of 128 positions, merged by
- *                         log-sum-exp.  `max_positions` fixes the launch shape (a captured graph can be
- *                         replayed while *pos advances up to max_positions - 1).
+ *                         {1,2,4,8}; split over the context in chunks of 64 positions, merged by
+ *                         log-sum-exp.  `max_positions` (<= 32768) fixes the launch shape (a captured
+ *                         graph can be replayed while *pos advances up to max_positions - 1).
+ *   kx_attn_decode_partial_bf16   the first stage only: the per-chunk results stay in the workspace for
+ *                         kx_gemv_awq_attn_merge_bf16 (below) to merge inside the o projection.
  *   kx_swiglu_bf16        out = bf16(silu(gate)) * up
  *   kx_add_bf16           out = a + b   (the reference's add operator, add_kernel.cu:4-12, in bf16)
  *   kx_embedding_bf16     out = table[*token, :]   (token clamped to the vocabulary)
@@ -189,6 +191,21 @@ size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head_dim, int32
 int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, uint16_t* out,
                         int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
                         int32_t max_positions, void* workspace, size_t workspace_bytes, void* stream);
+int kx_attn_decode_partial_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                                int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
+                                int32_t max_positions, void* workspace, size_t workspace_bytes, void* stream);
+/* The o projection of a decoder layer with the attention merge in its prologue (M = 1):
+ * y = attn W, where attn [n_q_heads * 128] is what kx_attn_decode_bf16 would have written, merged
+ * here from the workspace that kx_attn_decode_partial_bf16 filled with the same n_q_heads, n_kv_heads
+ * and max_positions.  Bitwise the result of kx_attn_decode_bf16 followed by kx_gemv_awq_bf16 on the
+ * vector kernel.  max_positions <= 5120 (80 chunks: a thread holds a row's per-chunk values in
+ * registers); longer contexts use the two separate calls.
+ * Replaces: the tail of LayerMHA + LayerMatmul back to back (kuiper/include/op/layer.h:8-20). */
+int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t attn_workspace_bytes, int32_t n_q_heads,
+                                int32_t n_kv_heads, int32_t head_dim, int32_t max_positions,
+                                const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
+                                uint16_t* y, int32_t N, int32_t group_size, void* workspace,
+                                size_t workspace_bytes, void* stream);
 int kx_swiglu_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int32_t n, void* stream);
 int kx_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int32_t n, void* stream);
 int kx_embedding_bf16(const uint16_t* table, const int32_t* token, uint16_t* out, int32_t vocab, int32_t dim,

@@ -36,6 +36,9 @@ SIGNATURES = {
                                             ctypes.c_float, _P]),
     "kx_attn_decode_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kx_attn_decode_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _SZ, _P]),
+    "kx_attn_decode_partial_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _SZ, _P]),
+    "kx_gemv_awq_attn_merge_bf16": (ctypes.c_int, [_P, _SZ, _I32, _I32, _I32, _I32, _P, _P, _P, _P, _I32, _I32, _P,
+                                                   _SZ, _P]),
     "kx_swiglu_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _P]),
     "kx_add_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _P]),
     "kx_embedding_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _P]),
@@ -194,6 +197,24 @@ def attn_decode_workspace(n_q, max_positions, device="cuda"):
 def attn_decode_bf16(q, k_cache, v_cache, out, n_q, n_kv, pos, max_positions, workspace):
     _check(load().kx_attn_decode_bf16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), n_q, n_kv, 128, _ptr(pos),
                                       max_positions, _ptr(workspace), workspace.numel(), _stream()))
+
+
+def attn_decode_partial_bf16(q, k_cache, v_cache, n_q, n_kv, pos, max_positions, workspace):
+    """First attention stage only; the per-chunk results stay in `workspace`."""
+    _check(load().kx_attn_decode_partial_bf16(_ptr(q), _ptr(k_cache), _ptr(v_cache), n_q, n_kv, 128, _ptr(pos),
+                                              max_positions, _ptr(workspace), workspace.numel(), _stream()))
+
+
+def gemv_awq_attn_merge_bf16(attn_workspace, n_q, n_kv, max_positions, qweight, scales, qzeros, y, group_size,
+                             workspace):
+    """y = (attention output merged from `attn_workspace`) W, one row."""
+    _check(load().kx_gemv_awq_attn_merge_bf16(_ptr(attn_workspace), attn_workspace.numel(), n_q, n_kv, 128,
+                                              max_positions, _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
+                                              y.shape[-1], group_size, _ptr(workspace),
+                                              0 if workspace is None else workspace.numel(), _stream()))
+
+
+FUSED_MERGE_MAX_POSITIONS = 80 * 64  # the o projection merges at most 80 chunks of 64 positions
 
 
 def swiglu_bf16(gate, up, out):

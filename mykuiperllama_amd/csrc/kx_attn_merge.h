@@ -1,0 +1,75 @@
+// Log-sum-exp merge of the per-chunk results of the flash-decoding kernel, shared by the stand-alone
+// merge kernel and by the prologue of the o-projection GEMV so that both produce the same bits.
+//
+// Per KV head the first stage leaves, for every chunk c of the context and each of its G query heads:
+//   part_out[kvh][c][g][0..127]   the unnormalised weighted sum of V rows, relative to the chunk maximum
+//   part_ml [kvh][c][g][0..1]     the chunk maximum m_c and the chunk sum of exponentials l_c (0: empty chunk)
+// The merged head is  sum_c part_out[c] * f_c / sum_c l_c * f_c  with  f_c = exp(m_c - max_c m_c).
+#ifndef KX_ATTN_MERGE_H
+#define KX_ATTN_MERGE_H
+
+#include <math.h>
+
+#include "kx_common.h"
+
+namespace kx {
+
+constexpr int kAttnChunk = 64;      // cache positions per chunk of the first stage
+constexpr int kMergeParts = 4;      // a dimension is summed over the chunks c = p, p + 4, ... for p = 0..3 side by side
+constexpr int kMergeBatch = 8;      // loads in flight per thread in the stand-alone merge
+constexpr int kMergeLanesLong = 8;  // chunks per lane the stand-alone merge provides for: 512 chunks
+
+// Chunk statistics of head (kvh, g) as one wave holds them: lane i has chunks i, i + 64, ...
+// (PER_LANE of them; chunks past nchunks read as empty).  Loading and finishing are separate so
+// that a caller can put other loads between the two.
+template <int PER_LANE>
+struct MergeStats {
+    float m[PER_LANE];
+    float l[PER_LANE];
+};
+
+template <int PER_LANE>
+__device__ __forceinline__ MergeStats<PER_LANE> attn_merge_load(const float* __restrict__ ml, int g, int G,
+                                                               int nchunks, int lane) {
+    MergeStats<PER_LANE> st;
+#pragma unroll
+    for (int u = 0; u < PER_LANE; u++) {
+        const int c = lane + u * kWave;
+        const int cc = c < nchunks ? c : nchunks - 1;  // clamped: the loads are straight-line code
+        const float mc = ml[(static_cast<size_t>(cc) * G + g) * 2];
+        const float lc = ml[(static_cast<size_t>(cc) * G + g) * 2 + 1];
+        st.m[u] = c < nchunks ? mc : -INFINITY;
+        st.l[u] = c < nchunks ? lc : 0.0f;
+    }
+    return st;
+}
+
+// Writes the factor of every chunk to s_factor[0 .. nchunks) and returns the normaliser, the same
+// value in every lane.  The result does not depend on PER_LANE (absent chunks are neutral).
+template <int PER_LANE>
+__device__ __forceinline__ float attn_merge_finish(const MergeStats<PER_LANE>& st, int nchunks, float* s_factor,
+                                                   int lane) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < PER_LANE; u++) m = fmaxf(m, st.m[u]);
+    m = wave_max(m);
+    float l = 0.0f;
+#pragma unroll
+    for (int u = 0; u < PER_LANE; u++) {
+        const int c = lane + u * kWave;
+        const float f = st.l[u] > 0.0f ? expf(st.m[u] - m) : 0.0f;  // chunks past the context have l == 0
+        if (c < nchunks) s_factor[c] = f;
+        l += st.l[u] * f;
+    }
+    return wave_sum(l);
+}
+
+// acc <- acc + v * f for a chunk that holds something; the partial sums of an empty chunk were never
+// written and are not looked at
+__device__ __forceinline__ float attn_merge_step(float acc, float v, float f) {
+    return __builtin_fmaf(f > 0.0f ? v : 0.0f, f, acc);
+}
+
+}  // namespace kx
+
+#endif  // KX_ATTN_MERGE_H

@@ -51,7 +51,7 @@ inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     return p;
 }
 
-inline AwqPlan make_valu_plan(int M, int K, int N) {
+inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true) {
     AwqPlan p;
     p.mfma = false;
     p.coltiles = (N / 8 + kWC - 1) / kWC;
@@ -66,7 +66,7 @@ inline AwqPlan make_valu_plan(int M, int K, int N) {
     // lane (512 rows of K per workgroup): all workgroups are resident at once and half as many
     // partial sums are exchanged.  Measured on the fused gate/up shape (4096 -> 24576): 15.7 -> 13.8 us.
     constexpr int kRowsLong = 8 * kSlotsPerWave * 32;
-    if (K % kRowsLong == 0 && static_cast<long>(p.coltiles) * (K / kRowsLong) >= 768) {
+    if (allow_long_rows && K % kRowsLong == 0 && static_cast<long>(p.coltiles) * (K / kRowsLong) >= 768) {
         p.rt = 32;
         p.ktiles = K / kRowsLong;
         return p;
@@ -355,5 +355,44 @@ extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_
         kx::launch_qkv<kx::kProAddNormLong>(p, fi, rope, qweight, scales, qzeros, partials, counters, K, N,
                                             group_size, kx::as_stream(stream));
     }
+    return kx::launch_status();
+}
+
+extern "C" int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t attn_workspace_bytes,
+                                           int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim,
+                                           int32_t max_positions, const int32_t* qweight, const uint16_t* scales,
+                                           const int32_t* qzeros, uint16_t* y, int32_t N, int32_t group_size,
+                                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (!attn_workspace) return KX_ERR_NULL_POINTER;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || (n_q_heads % n_kv_heads) != 0 ||
+        max_positions < 1) {
+        return KX_ERR_BAD_SHAPE;
+    }
+    const int K = n_q_heads * kx::kHeadDim;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, y, 1, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    const int nchunks = (max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    // a thread holds kMergeHold values of each of its elements: longer contexts take the separate merge
+    if (nchunks > kx::kMergeParts * kx::kMergeHold) return KX_ERR_BAD_SHAPE;
+    const size_t need = static_cast<size_t>(nchunks) * n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
+    if (attn_workspace_bytes < need) return KX_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(attn_workspace) % 16) return KX_ERR_ALIGNMENT;
+    kx::AwqPlan p = kx::make_valu_plan(1, K, N, false);
+    p.mb = 1;
+    p.mtiles = 1;
+    float* partials = nullptr;
+    uint32_t* counters = nullptr;
+    rc = kx::resolve_workspace(p, 1, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
+    kx::FusedInput fi{};
+    fi.part_out = static_cast<const float*>(attn_workspace);
+    fi.part_ml = fi.part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
+    fi.nchunks = nchunks;
+    fi.heads_per_kv = n_q_heads / n_kv_heads;
+    hipStream_t s = kx::as_stream(stream);
+#define KX_ARGS nullptr, qweight, scales, qzeros, y, partials, counters, 1, K, N, group_size, p.coltiles, p.ktiles, 1, s, fi
+    if (p.waves == 8) kx::launch_awq_gemv<8, 16, 1, kx::kProAttnMerge>(KX_ARGS);
+    else kx::launch_awq_gemv<4, 16, 1, kx::kProAttnMerge>(KX_ARGS);  // K = 128: one head
+#undef KX_ARGS
     return kx::launch_status();
 }

@@ -20,6 +20,7 @@
 #ifndef KX_AWQ_GEMV_KERNEL_H
 #define KX_AWQ_GEMV_KERNEL_H
 
+#include "kx_attn_merge.h"
 #include "kx_common.h"
 #include "kx_rope.h"
 #include "kx_splitk_exchange.h"
@@ -64,7 +65,10 @@ constexpr int kProNone = 0;     // x is a bf16 [M, K] tensor
 constexpr int kProSwiGLU = 1;   // x[m,k] = bf16( bf16(silu(a[m,k])) * b[m,k] )
 constexpr int kProAddNorm = 2;  // r = bf16(a + b) (b optional), x = gain * bf16(r * rsqrt(mean(r^2) + eps))
 constexpr int kProAddNormLong = 3;  // the same for rows of more than eight elements per thread
+constexpr int kProAttnMerge = 4;  // x = the attention output, merged here from the per-chunk results (M = 1)
 constexpr int kNormChunks = 2;  // most 16-byte pieces of a row a thread holds for the sum of squares
+constexpr int kMergeHold = 20;  // per-chunk values a thread holds per element it merges: 80 chunks in four parts
+constexpr int kMergeStatsPerLane = 2;  // chunks per lane of the wave that prepares a head's factors (>= 80 / 64)
 
 struct FusedInput {
     const uint16_t* a;     // gate, or the residual stream
@@ -73,6 +77,11 @@ struct FusedInput {
     uint16_t* r_out;       // where the updated residual stream goes (may be null); must not alias a
     int ld;                // elements between consecutive activation rows of a and b
     float eps;
+    // kProAttnMerge: results of the first attention stage (layout in kx_attn_merge.h)
+    const float* part_out;
+    const float* part_ml;
+    int nchunks;
+    int heads_per_kv;
 };
 
 constexpr float kCodeOffset = 16.0f;
@@ -116,12 +125,20 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     constexpr bool STAGED = PRO != kProNone;
     constexpr bool NORM = PRO == kProAddNorm || PRO == kProAddNormLong;
     constexpr int NCH = PRO == kProAddNormLong ? kNormChunks : 1;
+    constexpr bool MERGE = PRO == kProAttnMerge;
+    constexpr int HB = KB / kHeadDim > 0 ? KB / kHeadDim : 1;     // heads in the workgroup's K range
+    constexpr int EPT = kMergeParts * KB / THREADS;               // (part, row) elements a thread merges
+    static_assert(!MERGE || (MB == 1 && KB % kHeadDim == 0 && EPT * THREADS == kMergeParts * KB && HB <= WAVES),
+                  "the attention merge serves one activation row and whole heads");
     static_assert(RT % 8 == 0, "a lane reads its activations in 16-byte pieces");
     static_assert(KB <= THREADS, "one staging thread per row of the workgroup's K range");
 
     __shared__ __attribute__((aligned(16))) float red[WAVES][kTileCols];
     __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? MB : 1][STAGED ? KB : 8];  // staged activations, bf16
     __shared__ float s_ss[NORM ? MB : 1][WAVES];
+    __shared__ float s_factor[MERGE ? HB : 1][MERGE ? kMergeParts * kMergeHold : 1];
+    __shared__ float s_norm[MERGE ? HB : 1];
+    __shared__ float s_mpart[MERGE ? kMergeParts : 1][MERGE ? KB : 1];
 
     const int tid = threadIdx.x;
     const int ct = blockIdx.x % coltiles;
@@ -152,7 +169,37 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const uint16_t* b_src = has_b ? fi.b : fi.a;  // without a delta the second operand is read and ignored
     uint16_t own_a[MB], own_b[MB], own_gain = 0;
     uint4 row_a[NORM ? MB : 1][NCH], row_b[NORM ? MB : 1][NCH];
-    if constexpr (STAGED) {
+    float held[MERGE ? EPT : 1][MERGE ? kMergeHold : 1];
+    MergeStats<kMergeStatsPerLane> stats;
+    if constexpr (MERGE) {
+        // element e of the workgroup = (part, row): row of the K range, chunks part, part + 4, ...
+        const int G = fi.heads_per_kv;
+        const size_t cstride = static_cast<size_t>(G) * kHeadDim;
+#pragma unroll
+        for (int i = 0; i < EPT; i++) {
+            const int e = tid + i * THREADS;
+            const int part = e / KB;
+            const int rrow = kt * KB + e % KB;
+            const int row_c = rrow < K ? rrow : K - 1;
+            const int hq = row_c / kHeadDim;
+            const float* po = fi.part_out + (static_cast<size_t>(hq / G) * fi.nchunks * G + hq % G) * kHeadDim +
+                              row_c % kHeadDim;
+#pragma unroll
+            for (int j = 0; j < kMergeHold; j++) {
+                const int c = part + j * kMergeParts;
+                held[i][j] = po[(c < fi.nchunks ? c : fi.nchunks - 1) * cstride];
+            }
+        }
+        // wave w prepares the factors of head w of the K range
+        const int wave_id = tid / kWave;
+        if (wave_id < HB) {
+            const int hq0 = kt * HB + wave_id;
+            const int hq = hq0 * kHeadDim < K ? hq0 : K / kHeadDim - 1;
+            stats = attn_merge_load<kMergeStatsPerLane>(fi.part_ml + static_cast<size_t>(hq / G) * fi.nchunks * G * 2,
+                                                        hq % G, G, fi.nchunks, tid % kWave);
+        }
+    }
+    if constexpr (STAGED && !MERGE) {
         const int krow_c = krow < K ? krow : K - 1;
 #pragma unroll
         for (int m = 0; m < MB; m++) {
@@ -214,6 +261,35 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    if constexpr (MERGE) {
+        const int wave_id = tid / kWave;
+        if (wave_id < HB) {
+            const float l = attn_merge_finish<kMergeStatsPerLane>(stats, fi.nchunks, s_factor[wave_id], tid % kWave);
+            if (tid % kWave == 0) s_norm[wave_id] = l;
+        }
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < EPT; i++) {
+            const int e = tid + i * THREADS;
+            const int part = e / KB;
+            const int row = e % KB;
+            const float* f = s_factor[row / kHeadDim];
+            float acc_m = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kMergeHold; j++) {
+                const int c = part + j * kMergeParts;
+                if (c < fi.nchunks) acc_m = attn_merge_step(acc_m, held[i][j], f[c]);
+            }
+            s_mpart[part][row] = acc_m;
+        }
+        lds_barrier();
+        if (tid < KB) {
+            const float total = (s_mpart[0][tid] + s_mpart[1][tid]) + (s_mpart[2][tid] + s_mpart[3][tid]);
+            const uint16_t xv = f32_to_bf16(total / s_norm[tid / kHeadDim]);
+            s_x[0][tid] = stager ? xv : static_cast<uint16_t>(0);
+        }
+        lds_barrier();
+    }
     if constexpr (PRO == kProSwiGLU) {
         if (tid < KB) {
 #pragma unroll

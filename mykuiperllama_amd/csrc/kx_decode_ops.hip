@@ -7,6 +7,7 @@
 // LayerSwiGLU, LayerAdd, LayerEmbedding: kuiper/include/op/layer.h:8-20) and names their scratch
 // buffers (model::ModelBufferType, kuiper/include/base/base.h:12-31) but implements none of them
 // except the fp32 add (kuiper/source/op/kernel/cuda/add_kernel.cu:4-12).
+#include "kx_attn_merge.h"
 #include "kx_common.h"
 #include "kx_rope.h"
 
@@ -126,7 +127,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 // G heads the unnormalised 128-vector, the chunk maximum and the chunk sum of exponentials.
 // Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
 // ------------------------------------------------------------------------------------------------
-constexpr int kAttnChunk = 64;
 constexpr int kAttnThreads = 256;
 constexpr int kAttnSlots = kAttnThreads / 16;  // cache positions a workgroup handles side by side
 constexpr int kAccHeads = 4;                   // heads whose slot sums fit in LDS together (32 KiB)
@@ -279,7 +279,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     }
 }
 
-constexpr int kMergeParts = 4;  // chunk subsets summed side by side
 constexpr int kMergeThreads = kHeadDim * kMergeParts;
 
 template <int G>
@@ -287,74 +286,43 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
                                                                     const float* __restrict__ part_ml,
                                                                     uint16_t* __restrict__ out, int nchunks) {
     extern __shared__ float s_factor[];  // nchunks rescaling factors exp(m_c - m)
-    __shared__ float s_red[kMergeThreads / kWave];
+    __shared__ float s_norm;
     __shared__ float s_part[kMergeParts][kHeadDim];
     const int head = blockIdx.x;  // query head
     const int kvh = head / G;
     const int g = head % G;
     const int tid = threadIdx.x;
-    const float* ml = part_ml + static_cast<size_t>(kvh) * nchunks * G * 2;
-
-    // chunk maxima and sums, one chunk per thread at a time; both loads go out together
-    float mc_keep = -INFINITY, lc_keep = 0.0f;  // the thread's first chunk stays in registers
-    float m = -INFINITY;
-    for (int c = tid; c < nchunks; c += kMergeThreads) {
-        const float mc = ml[(static_cast<size_t>(c) * G + g) * 2];
-        const float lc = ml[(static_cast<size_t>(c) * G + g) * 2 + 1];
-        if (c == tid) {
-            mc_keep = mc;
-            lc_keep = lc;
-        }
-        m = fmaxf(m, mc);
+    if (tid < kWave) {
+        const MergeStats<kMergeLanesLong> st =
+            attn_merge_load<kMergeLanesLong>(part_ml + static_cast<size_t>(kvh) * nchunks * G * 2, g, G, nchunks, tid);
+        const float l = attn_merge_finish<kMergeLanesLong>(st, nchunks, s_factor, tid);
+        if (tid == 0) s_norm = l;
     }
-    m = wave_max(m);
-    if (tid % kWave == 0) s_red[tid / kWave] = m;
     __syncthreads();
-    m = s_red[0];
-#pragma unroll
-    for (int w = 1; w < kMergeThreads / kWave; w++) m = fmaxf(m, s_red[w]);
-    __syncthreads();
-    float l = 0.0f;
-    for (int c = tid; c < nchunks; c += kMergeThreads) {
-        const float mc = c == tid ? mc_keep : ml[(static_cast<size_t>(c) * G + g) * 2];
-        const float lc = c == tid ? lc_keep : ml[(static_cast<size_t>(c) * G + g) * 2 + 1];
-        const float f = lc > 0.0f ? expf(mc - m) : 0.0f;  // chunks past the context have lc == 0
-        s_factor[c] = f;
-        l += lc * f;
-    }
-    l = wave_sum(l);
-    if (tid % kWave == 0) s_red[tid / kWave] = l;
-    __syncthreads();
-    l = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kMergeThreads / kWave; w++) l += s_red[w];
 
-    // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...; eight loads in flight
+    // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...
     const int d = tid % kHeadDim;
     const int part = tid / kHeadDim;
     const float* po = part_out + (static_cast<size_t>(kvh) * nchunks * G + g) * kHeadDim + d;
     const size_t cstride = static_cast<size_t>(G) * kHeadDim;
     float acc = 0.0f;
-    for (int c0 = part; c0 < nchunks; c0 += 8 * kMergeParts) {
-        float v[8];
+    for (int c0 = part; c0 < nchunks; c0 += kMergeBatch * kMergeParts) {
+        float v[kMergeBatch];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < kMergeBatch; u++) {
             const int c = c0 + u * kMergeParts;
             v[u] = (c < nchunks && s_factor[c] > 0.0f) ? po[c * cstride] : 0.0f;
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < kMergeBatch; u++) {
             const int c = c0 + u * kMergeParts;
-            if (c < nchunks) acc = __builtin_fmaf(v[u], s_factor[c], acc);
+            if (c < nchunks) acc = attn_merge_step(acc, v[u], s_factor[c]);
         }
     }
     s_part[part][d] = acc;
     __syncthreads();
     if (part == 0) {
-        float total = 0.0f;
-#pragma unroll
-        for (int q = 0; q < kMergeParts; q++) total += s_part[q][d];
-        out[static_cast<size_t>(head) * kHeadDim + d] = f32_to_bf16(total / l);
+        out[static_cast<size_t>(head) * kHeadDim + d] = f32_to_bf16(((s_part[0][d] + s_part[1][d]) + (s_part[2][d] + s_part[3][d])) / s_norm);
     }
 }
 
@@ -510,11 +478,12 @@ extern "C" size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head
     return nchunks * n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
 }
 
-extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
-                                   uint16_t* out, int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim,
-                                   const int32_t* pos, int32_t max_positions, void* workspace,
-                                   size_t workspace_bytes, void* stream) {
-    if (!q || !k_cache || !v_cache || !out || !pos || !workspace) return KX_ERR_NULL_POINTER;
+namespace {
+// Shared by the two attention entry points: checks, then the first stage and (with `out`) the merge.
+int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, uint16_t* out,
+                int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos, int32_t max_positions,
+                void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k_cache || !v_cache || !pos || !workspace) return KX_ERR_NULL_POINTER;
     if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || (n_q_heads % n_kv_heads) != 0 ||
         max_positions < 1) {
         return KX_ERR_BAD_SHAPE;
@@ -526,19 +495,40 @@ extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, c
         return KX_ERR_ALIGNMENT;
     }
     const int nchunks = (max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    if (nchunks > kx::kMergeLanesLong * kx::kWave) return KX_ERR_BAD_SHAPE;  // 32768 positions
     float* part_out = static_cast<float*>(workspace);
     float* part_ml = part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
     const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
     hipStream_t s = kx::as_stream(stream);
     dim3 grid1(nchunks, n_kv_heads);
-#define KX_ATTN(GG)                                                                                           \
-    hipLaunchKernelGGL((kx::attn_decode_stage1<GG>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache, v_cache, \
-                       part_out, part_ml, n_kv_heads, pos, nchunks, max_positions, scale);                                    \
-    hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kMergeThreads),               \
-                       nchunks * sizeof(float), s, part_out, part_ml, out, nchunks)
-    if (G == 1) { KX_ATTN(1); } else if (G == 2) { KX_ATTN(2); } else if (G == 4) { KX_ATTN(4); } else { KX_ATTN(8); }
+#define KX_ATTN(GG)                                                                                             \
+    hipLaunchKernelGGL((kx::attn_decode_stage1<GG>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache, v_cache,  \
+                       part_out, part_ml, n_kv_heads, pos, nchunks, max_positions, scale);                      \
+    if (out) {                                                                                                  \
+        hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kMergeThreads),              \
+                           nchunks * sizeof(float), s, part_out, part_ml, out, nchunks);                        \
+    }
+    if (G == 1) { KX_ATTN(1) } else if (G == 2) { KX_ATTN(2) } else if (G == 4) { KX_ATTN(4) } else { KX_ATTN(8) }
 #undef KX_ATTN
     return kx::launch_status();
+}
+}  // namespace
+
+extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                                   uint16_t* out, int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim,
+                                   const int32_t* pos, int32_t max_positions, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+    if (!out) return KX_ERR_NULL_POINTER;
+    return attn_decode(q, k_cache, v_cache, out, n_q_heads, n_kv_heads, head_dim, pos, max_positions, workspace,
+                       workspace_bytes, stream);
+}
+
+extern "C" int kx_attn_decode_partial_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                                           int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim,
+                                           const int32_t* pos, int32_t max_positions, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
+    return attn_decode(q, k_cache, v_cache, nullptr, n_q_heads, n_kv_heads, head_dim, pos, max_positions, workspace,
+                       workspace_bytes, stream);
 }
 
 extern "C" int kx_swiglu_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int32_t n, void* stream) {

@@ -15,8 +15,9 @@ packed tensors of the separate projections are concatenated along N when the wei
 (rows are laid end to end; the nibble order inside a word is untouched).  The residual add is fused
 into the next RMSNorm, and by default (`fused=True`) both ride in the prologue of the GEMV that
 consumes the normalised row, as does SwiGLU in front of the down projection, and the per-head
-norm, rotation and cache append ride in the epilogue of the q/k/v GEMV: six launches per layer
-instead of ten.  The residual stream then alternates between two buffers, because a fused
+norm, rotation and cache append ride in the epilogue of the q/k/v GEMV, and the o projection
+merges the chunks of the attention itself (contexts up to 5120 positions): five launches per
+layer instead of ten.  The residual stream then alternates between two buffers, because a fused
 launch reads the whole incoming row in every workgroup while it writes the updated one.
 Every launch goes to torch's current stream, so a step can be captured in a HIP graph; token and
 position live in device memory for that reason.
@@ -171,9 +172,16 @@ class DecodeModel:
             capi.gemv_awq_qkv_rope_bf16(xa, None if li == 0 else self.down, L["in_norm"], c.eps, xb, qw, sc, qz,
                                         L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
                                         c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps, g, ws)
-            capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
-                                  self.max_positions, self.attn_ws)
-            self._awq(self.attn, L["o"], self.o)
+            if self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS:
+                capi.attn_decode_partial_bf16(self.q, self.k_cache[li], self.v_cache[li], c.n_q, c.n_kv, self.pos,
+                                              self.max_positions, self.attn_ws)
+                qw, sc, qz = L["o"]
+                capi.gemv_awq_attn_merge_bf16(self.attn_ws, c.n_q, c.n_kv, self.max_positions, qw, sc, qz, self.o,
+                                              g, ws)
+            else:
+                capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv,
+                                      self.pos, self.max_positions, self.attn_ws)
+                self._awq(self.attn, L["o"], self.o)
             qw, sc, qz = L["gateup"]
             capi.gemv_awq_addnorm_bf16(xb, self.o, L["post_norm"], c.eps, xa, qw, sc, qz, self.gu, g, ws)
             qw, sc, qz = L["down"]
@@ -185,7 +193,10 @@ class DecodeModel:
             capi.argmax_bf16(self.logits, self.next_token)
 
     def launches_per_step(self, with_lm_head=True, fused=True):
-        return 1 + self.cfg.layers * (6 if fused else 10) + 1 + (2 if with_lm_head else 0)
+        per_layer = 10
+        if fused:
+            per_layer = 5 if self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS else 6
+        return 1 + self.cfg.layers * per_layer + 1 + (2 if with_lm_head else 0)
 
 
 def step_bytes(cfg, ctx, with_lm_head=True):

@@ -233,6 +233,70 @@ def test_qkv_rope_launch_rejects_bad_arguments(capi, torch):
     assert e.value.code == -1
 
 
+MERGE_CASES = [
+    # n_q, n_kv, pos, max_positions, N, group
+    (32, 8, 4096, 4224, 4096, 128),   # Qwen3-8B at the benchmark's context
+    (32, 8, 0, 4224, 4096, 128),      # a single cached position
+    (32, 8, 63, 5120, 1024, 128),     # the longest context the merging projection takes
+    (64, 8, 1000, 1100, 5120, 128),   # eight query heads per KV head
+    (4, 2, 37, 48, 512, 128),
+    (2, 1, 100, 128, 264, 32),        # K = 256, ragged N
+    (1, 1, 5, 64, 64, 32),            # K = 128: four waves, one head
+    (4, 4, 127, 128, 256, 64),        # no grouping, context ends on a chunk boundary
+]
+
+
+@pytest.mark.parametrize("n_q,n_kv,pos_value,max_pos,N,group", MERGE_CASES)
+def test_attention_merge_in_the_o_projection_equals_separate_launches(capi, torch, n_q, n_kv, pos_value, max_pos, N,
+                                                                      group):
+    K = n_q * 128
+    _, (qw, sc, qz) = weights(torch, f"fused_merge_{n_q}_{n_kv}_{N}", 1, K, N, group)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(n_q * 1000 + pos_value)
+    q = torch.randn((n_q, 128), device="cuda", generator=g).bfloat16()
+    kc = torch.randn((max_pos, n_kv, 128), device="cuda", generator=g).bfloat16()
+    vc = torch.randn((max_pos, n_kv, 128), device="cuda", generator=g).bfloat16()
+    kc[pos_value + 1:] = float("nan")  # rows past the context must not matter
+    vc[pos_value + 1:] = float("nan")
+    pos = torch.tensor([pos_value], dtype=torch.int32, device="cuda")
+    ws = capi.make_workspace(1, K, N)
+
+    attn_ws = capi.attn_decode_workspace(n_q, max_pos)
+    attn_ws.view(torch.float32)[: attn_ws.numel() // 4].fill_(float("nan"))  # nothing stale may be read
+    attn = torch.empty((1, K), dtype=torch.bfloat16, device="cuda")
+    y_sep = torch.full((1, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.attn_decode_bf16(q, kc, vc, attn, n_q, n_kv, pos, max_pos, attn_ws)
+    capi.gemv_awq_bf16(attn, qw, sc, qz, y_sep, group, ws)
+
+    attn_ws2 = capi.attn_decode_workspace(n_q, max_pos)
+    attn_ws2.view(torch.float32)[: attn_ws2.numel() // 4].fill_(float("nan"))
+    y_one = torch.full((1, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.attn_decode_partial_bf16(q, kc, vc, n_q, n_kv, pos, max_pos, attn_ws2)
+    capi.gemv_awq_attn_merge_bf16(attn_ws2, n_q, n_kv, max_pos, qw, sc, qz, y_one, group, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y_sep.float()).all()
+    assert torch.equal(y_one.view(torch.int16), y_sep.view(torch.int16))
+
+
+def test_attention_merge_rejects_long_contexts_and_bad_arguments(capi, torch):
+    n_q, n_kv, N, group = 2, 1, 256, 128
+    _, (qw, sc, qz) = weights(torch, "fused_merge_bad", 1, n_q * 128, N, group)
+    y = torch.zeros((1, N), dtype=torch.bfloat16, device="cuda")
+    ws = capi.make_workspace(1, n_q * 128, N)
+    long_ws = capi.attn_decode_workspace(n_q, 5121)
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_attn_merge_bf16(long_ws, n_q, n_kv, 5121, qw, sc, qz, y, group, ws)
+    assert e.value.code == -2
+    small_ws = capi.attn_decode_workspace(n_q, 64)
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_attn_merge_bf16(small_ws, n_q, n_kv, 4096, qw, sc, qz, y, group, ws)
+    assert e.value.code == -3
+    rc = capi.load().kx_gemv_awq_attn_merge_bf16(None, 1 << 20, n_q, n_kv, 128, 64, qw.data_ptr(), sc.data_ptr(),
+                                                 qz.data_ptr(), y.data_ptr(), N, group, ws.data_ptr(), ws.numel(),
+                                                 None)
+    assert rc == -1
+
+
 def test_fused_launches_are_deterministic_and_leave_the_workspace_reusable(capi, torch):
     M, K, N, group = 1, 4096, 6144, 128
     _, (qw, sc, qz) = weights(torch, "fused_repeat", M, K, N, group)
