@@ -4,9 +4,10 @@
 //
 // The packed stream is consumed as it lies in memory: qweight int32 [K, N/8], one word = eight
 // columns of one row.  A lane owns one word column and RT consecutive rows (all inside one
-// quantisation group), so that zero point and scale are applied once per lane and column:
+// quantisation group), so that zero point and scale are applied once per lane and column.  Codes
+// enter the arithmetic as bf16 numbers 16 + q, two rows per dot-product instruction:
 //
-//   y_part[n] = s[g,n] * ( sum_r q[k0+r,n] * x[k0+r]  -  z[g,n] * sum_r x[k0+r] )
+//   y_part[n] = s[g,n] * ( sum_r (16 + q[k0+r,n]) * x[k0+r]  -  (16 + z[g,n]) * sum_r x[k0+r] )
 //
 // A wave covers 32 consecutive word columns (128 contiguous bytes of each row, 256 output
 // columns) times two row slots; a workgroup stacks WAVES waves along K.  Row slots meet in LDS.
@@ -35,10 +36,10 @@ constexpr int kSlotsPerWave = kWave / kWC;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-// The eight codes of a packed word as floats, indexed by column (0..7) inside the word.
-// A byte 0x0q read as OCP fp8 (e4m3) is exactly q * 2^-9 for every q in 0..15 (subnormal below
-// 8, normal from 8 on), so the packed fp8 -> fp32 conversion unpacks two codes per instruction.
-// The factor 2^-9 is undone by kCodeScale when the group scale is applied.
+// The eight codes of a packed word as floats times 2^-9, indexed by column (0..7) inside the word;
+// used for the zero points, once per lane.  A byte 0x0q read as OCP fp8 (e4m3) is exactly q * 2^-9
+// for every q in 0..15 (subnormal below 8, normal from 8 on), so the packed fp8 -> fp32 conversion
+// unpacks two codes per instruction; kCodeScale undoes the factor.
 constexpr float kCodeScale = 512.0f;
 
 __device__ __forceinline__ void unpack_codes(uint32_t w, float (&q)[8]) {
