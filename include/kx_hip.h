@@ -130,6 +130,86 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
                               size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Chained GEMV (M = 1): one launch whose activations come from the previous operator of a decoder
+ * layer and whose result goes straight into the next one.  `in_kind` selects where the activation
+ * row x [K] comes from, `out_kind` what happens to the finished row o [N]; only the fields of the
+ * selected kinds are read.
+ *
+ *   KX_IN_ROW       x                                    bf16 [K], 16-byte aligned
+ *   KX_IN_SWIGLU    gate, up                             x = bf16(bf16(silu(gate)) * up)
+ *   KX_IN_ATTN      attn_workspace (+ bytes), n_q_heads, n_kv_heads, max_positions
+ *                                                        x = attention output merged from the workspace
+ *                                                        of kx_attn_decode_partial_bf16 (K = n_q_heads * 128)
+ *   KX_IN_NORM      norm_row, norm_sumsq, norm_parts, norm_gain, norm_eps
+ *                                                        x = gain * bf16(row * rsqrt(sum(sumsq) / K + eps)),
+ *                                                        sumsq = the per-tile sums KX_OUT_RESIDUAL left
+ *   KX_OUT_ROW      y                                    y = bf16(o)
+ *   KX_OUT_RESIDUAL residual_in, residual_out, sumsq_out residual_out = bf16(residual_in + bf16(o)) (may be
+ *                                                        in place), sumsq_out[t] = sum of squares of columns
+ *                                                        256 t .. 256 t + 255 of residual_out, t < ceil(N / 256)
+ *   KX_OUT_QKV_ROPE q_gain, k_gain, q_out, k_cache, v_cache, pos, rope_n_q_heads, rope_n_kv_heads,
+ *                   rope_theta, qk_eps                   as kx_gemv_awq_qkv_rope_bf16 (N = (n_q + 2 n_kv) * 128)
+ *
+ * The sum of squares of KX_OUT_RESIDUAL / KX_IN_NORM is added tile by tile, an order of its own:
+ * results agree with kx_add_rmsnorm_bf16 followed by the GEMV to within the rounding of that sum
+ * (an occasional last-bit difference in the normalised row), not bit for bit.
+ * Always the vector kernel.  Replaces: the chain LayerMHA -> LayerMatmul -> LayerAdd -> LayerRMSNorm ->
+ * LayerMatmul -> LayerSwiGLU -> LayerMatmul -> LayerAdd -> LayerRMSNorm of a decoder layer, one link
+ * per call (slots kuiper/include/op/layer.h:8-20; none implemented in the reference).
+ * ------------------------------------------------------------------------------------------ */
+#define KX_IN_ROW 0
+#define KX_IN_SWIGLU 1
+#define KX_IN_ATTN 2
+#define KX_IN_NORM 3
+#define KX_OUT_ROW 0
+#define KX_OUT_RESIDUAL 1
+#define KX_OUT_QKV_ROPE 2
+
+typedef struct kx_chain_desc {
+    int32_t in_kind;
+    int32_t out_kind;
+    /* KX_IN_ROW */
+    const uint16_t* x;
+    /* KX_IN_SWIGLU */
+    const uint16_t* gate;
+    const uint16_t* up;
+    /* KX_IN_ATTN */
+    const void* attn_workspace;
+    size_t attn_workspace_bytes;
+    int32_t n_q_heads;
+    int32_t n_kv_heads;
+    int32_t max_positions;
+    /* KX_IN_NORM */
+    int32_t norm_parts;
+    const uint16_t* norm_row;
+    const float* norm_sumsq;
+    const uint16_t* norm_gain;
+    float norm_eps;
+    /* KX_OUT_QKV_ROPE (scalars) */
+    float rope_theta;
+    float qk_eps;
+    int32_t rope_n_q_heads;
+    int32_t rope_n_kv_heads;
+    /* KX_OUT_ROW */
+    uint16_t* y;
+    /* KX_OUT_RESIDUAL */
+    const uint16_t* residual_in;
+    uint16_t* residual_out;
+    float* sumsq_out;
+    /* KX_OUT_QKV_ROPE (pointers) */
+    const uint16_t* q_gain;
+    const uint16_t* k_gain;
+    uint16_t* q_out;
+    uint16_t* k_cache;
+    uint16_t* v_cache;
+    const int32_t* pos;
+} kx_chain_desc;
+
+int kx_gemv_awq_chain_bf16(const kx_chain_desc* desc, const int32_t* qweight, const uint16_t* scales,
+                           const int32_t* qzeros, int32_t K, int32_t N, int32_t group_size, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * BF16 GEMV fallback (non-quantised layers, lm_head):   y[m,n] = sum_k x[m,k] * W[n,k]
  *   W bf16 [N,K] row-major (dim0 = output features, dim1 = input features, the reading of
  *   LayerParam weights as [dim0, dim1]: kuiper/source/op/layer.cpp:256-276), K a multiple of 8,

@@ -29,6 +29,7 @@ SIGNATURES = {
     "kx_gemv_awq_qkv_rope_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _P, _P, _P, _P,
                                                  _I32, _I32, _I32, _P, ctypes.c_float, ctypes.c_float, _I32, _I32,
                                                  _P, _SZ, _P]),
+    "kx_gemv_awq_chain_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "kx_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
     "kx_add_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
@@ -45,6 +46,27 @@ SIGNATURES = {
     "kx_argmax_bf16": (ctypes.c_int, [_P, _I32, _P, _P]),
     "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
 }
+
+
+class ChainDesc(ctypes.Structure):
+    """Mirror of kx_chain_desc (include/kx_hip.h), field for field."""
+    _fields_ = [
+        ("in_kind", _I32), ("out_kind", _I32),
+        ("x", _P),
+        ("gate", _P), ("up", _P),
+        ("attn_workspace", _P), ("attn_workspace_bytes", _SZ),
+        ("n_q_heads", _I32), ("n_kv_heads", _I32), ("max_positions", _I32),
+        ("norm_parts", _I32), ("norm_row", _P), ("norm_sumsq", _P), ("norm_gain", _P), ("norm_eps", ctypes.c_float),
+        ("rope_theta", ctypes.c_float), ("qk_eps", ctypes.c_float),
+        ("rope_n_q_heads", _I32), ("rope_n_kv_heads", _I32),
+        ("y", _P),
+        ("residual_in", _P), ("residual_out", _P), ("sumsq_out", _P),
+        ("q_gain", _P), ("k_gain", _P), ("q_out", _P), ("k_cache", _P), ("v_cache", _P), ("pos", _P),
+    ]
+
+
+IN_ROW, IN_SWIGLU, IN_ATTN, IN_NORM = 0, 1, 2, 3
+OUT_ROW, OUT_RESIDUAL, OUT_QKV_ROPE = 0, 1, 2
 
 
 class KxError(RuntimeError):
@@ -212,6 +234,16 @@ def gemv_awq_attn_merge_bf16(attn_workspace, n_q, n_kv, max_positions, qweight, 
                                               max_positions, _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
                                               y.shape[-1], group_size, _ptr(workspace),
                                               0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_awq_chain_bf16(desc, qweight, scales, qzeros, K, N, group_size, workspace):
+    """One link of a decoder layer's chain: see kx_chain_desc.  `desc` maps field names to tensors,
+    None or scalars; tensors are passed by address."""
+    d = ChainDesc()
+    for name, value in desc.items():
+        setattr(d, name, value.data_ptr() if hasattr(value, "data_ptr") else value)
+    _check(load().kx_gemv_awq_chain_bf16(ctypes.byref(d), _ptr(qweight), _ptr(scales), _ptr(qzeros), K, N, group_size,
+                                         _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream()))
 
 
 FUSED_MERGE_MAX_POSITIONS = 80 * 64  # the o projection merges at most 80 chunks of 64 positions

@@ -142,12 +142,12 @@ void launch_fused(const AwqPlan& p, const FusedInput& fi, const int32_t* qweight
 
 // Checks shared by every AWQ entry point; `x` stands for whichever tensors feed the activations.
 inline int check_awq_weights(const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
-                             const uint16_t* y, int M, int K, int N, int group_size) {
-    if (!qweight || !scales || !qzeros || !y) return KX_ERR_NULL_POINTER;
+                             const uint16_t* y, int M, int K, int N, int group_size, bool stores_y = true) {
+    if (!qweight || !scales || !qzeros || (stores_y && !y)) return KX_ERR_NULL_POINTER;
     if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8 || (N % 8) != 0) return KX_ERR_BAD_SHAPE;
     if (group_size < 32 || (group_size % 32) != 0 || (K % group_size) != 0) return KX_ERR_BAD_SHAPE;
     if (reinterpret_cast<uintptr_t>(scales) % 16 || reinterpret_cast<uintptr_t>(qweight) % 4 ||
-        reinterpret_cast<uintptr_t>(qzeros) % 4 || reinterpret_cast<uintptr_t>(y) % 8) {
+        reinterpret_cast<uintptr_t>(qzeros) % 4 || (stores_y && reinterpret_cast<uintptr_t>(y) % 8)) {
         return KX_ERR_ALIGNMENT;
     }
     return KX_OK;
@@ -394,5 +394,154 @@ extern "C" int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t at
     if (p.waves == 8) kx::launch_awq_gemv<8, 16, 1, kx::kProAttnMerge>(KX_ARGS);
     else kx::launch_awq_gemv<4, 16, 1, kx::kProAttnMerge>(KX_ARGS);  // K = 128: one head
 #undef KX_ARGS
+    return kx::launch_status();
+}
+
+namespace kx {
+namespace {
+
+template <int PRO, int EPI>
+void launch_chain(const AwqPlan& p, const FusedInput& fi, const RopeTarget& rope, const ResidualTarget& res,
+                  const uint16_t* x, const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
+                  uint16_t* y, float* partials, uint32_t* counters, int K, int N, int group, hipStream_t stream) {
+#define KX_ARGS x, qweight, scales, qzeros, y, partials, counters, 1, K, N, group, p.coltiles, p.ktiles, 1, stream, fi, rope, res
+    if constexpr (PRO != kProAttnMerge) {
+        if (p.rt == 32) {
+            launch_awq_gemv<8, 32, 1, PRO, EPI>(KX_ARGS);
+            return;
+        }
+    }
+    if (p.waves == 8) launch_awq_gemv<8, 16, 1, PRO, EPI>(KX_ARGS);
+    else if (p.rt == 16) launch_awq_gemv<4, 16, 1, PRO, EPI>(KX_ARGS);
+    else if constexpr (PRO != kProAttnMerge) launch_awq_gemv<4, 8, 1, PRO, EPI>(KX_ARGS);
+#undef KX_ARGS
+}
+
+}  // namespace
+}  // namespace kx
+
+extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qweight, const uint16_t* scales,
+                                      const int32_t* qzeros, int32_t K, int32_t N, int32_t group_size,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+    if (!d) return KX_ERR_NULL_POINTER;
+    kx::FusedInput fi{};
+    kx::RopeTarget rope{};
+    kx::ResidualTarget res{};
+    const uint16_t* x = nullptr;
+    uint16_t* y = nullptr;
+    bool long_rows = true;
+
+    // where the activations come from
+    switch (d->in_kind) {
+        case KX_IN_ROW:
+            if (!d->x) return KX_ERR_NULL_POINTER;
+            if (reinterpret_cast<uintptr_t>(d->x) % 16) return KX_ERR_ALIGNMENT;
+            x = d->x;
+            break;
+        case KX_IN_SWIGLU:
+            if (!d->gate || !d->up) return KX_ERR_NULL_POINTER;
+            if (reinterpret_cast<uintptr_t>(d->gate) % 2 || reinterpret_cast<uintptr_t>(d->up) % 2) return KX_ERR_ALIGNMENT;
+            fi.a = d->gate;
+            fi.b = d->up;
+            fi.ld = K;
+            break;
+        case KX_IN_ATTN: {
+            if (!d->attn_workspace) return KX_ERR_NULL_POINTER;
+            if (d->n_q_heads < 1 || d->n_kv_heads < 1 || (d->n_q_heads % d->n_kv_heads) != 0 || d->max_positions < 1 ||
+                K != d->n_q_heads * kx::kHeadDim) {
+                return KX_ERR_BAD_SHAPE;
+            }
+            const int nchunks = (d->max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+            if (nchunks > kx::kMergeParts * kx::kMergeHold) return KX_ERR_BAD_SHAPE;
+            const size_t need = static_cast<size_t>(nchunks) * d->n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
+            if (d->attn_workspace_bytes < need) return KX_ERR_WORKSPACE;
+            if (reinterpret_cast<uintptr_t>(d->attn_workspace) % 16) return KX_ERR_ALIGNMENT;
+            fi.part_out = static_cast<const float*>(d->attn_workspace);
+            fi.part_ml = fi.part_out + static_cast<size_t>(nchunks) * d->n_q_heads * kx::kHeadDim;
+            fi.nchunks = nchunks;
+            fi.heads_per_kv = d->n_q_heads / d->n_kv_heads;
+            long_rows = false;  // the merge covers at most 256 rows of K per workgroup
+            break;
+        }
+        case KX_IN_NORM:
+            if (!d->norm_row || !d->norm_sumsq || !d->norm_gain) return KX_ERR_NULL_POINTER;
+            if (d->norm_parts != (K + kx::kTileCols - 1) / kx::kTileCols || d->norm_parts > kx::kWave) return KX_ERR_BAD_SHAPE;
+            if (reinterpret_cast<uintptr_t>(d->norm_row) % 2 || reinterpret_cast<uintptr_t>(d->norm_sumsq) % 4 ||
+                reinterpret_cast<uintptr_t>(d->norm_gain) % 2) {
+                return KX_ERR_ALIGNMENT;
+            }
+            fi.a = d->norm_row;
+            fi.gain = d->norm_gain;
+            fi.eps = d->norm_eps;
+            fi.sumsq = d->norm_sumsq;
+            fi.sumsq_parts = d->norm_parts;
+            fi.ld = K;
+            break;
+        default: return KX_ERR_BAD_SHAPE;
+    }
+
+    // where the result goes
+    const uint16_t* out_probe = nullptr;  // any output pointer, for the shared checks
+    switch (d->out_kind) {
+        case KX_OUT_ROW:
+            if (!d->y) return KX_ERR_NULL_POINTER;
+            y = d->y;
+            out_probe = d->y;
+            break;
+        case KX_OUT_RESIDUAL:
+            if (!d->residual_in || !d->residual_out || !d->sumsq_out) return KX_ERR_NULL_POINTER;
+            if (reinterpret_cast<uintptr_t>(d->residual_in) % 2 || reinterpret_cast<uintptr_t>(d->residual_out) % 2 ||
+                reinterpret_cast<uintptr_t>(d->sumsq_out) % 4) {
+                return KX_ERR_ALIGNMENT;
+            }
+            // the norm prologue reads all of its row while this epilogue would be rewriting it
+            if (d->in_kind == KX_IN_NORM && d->residual_out == d->norm_row) return KX_ERR_ALIAS;
+            res.in = d->residual_in;
+            res.out = d->residual_out;
+            res.sumsq = d->sumsq_out;
+            out_probe = d->residual_out;
+            break;
+        case KX_OUT_QKV_ROPE:
+            if (!d->q_gain || !d->k_gain || !d->q_out || !d->k_cache || !d->v_cache || !d->pos) return KX_ERR_NULL_POINTER;
+            if (d->rope_n_q_heads < 1 || d->rope_n_kv_heads < 1 || !(d->rope_theta > 1.0f) ||
+                N != (d->rope_n_q_heads + 2 * d->rope_n_kv_heads) * kx::kHeadDim ||
+                (d->rope_n_q_heads + 2 * d->rope_n_kv_heads) % (kx::kTileCols / kx::kHeadDim) != 0) {
+                return KX_ERR_BAD_SHAPE;
+            }
+            rope = kx::RopeTarget{d->q_gain, d->k_gain, d->q_out, d->k_cache, d->v_cache, d->pos,
+                                  d->rope_n_q_heads, d->rope_n_kv_heads, log2f(d->rope_theta), d->qk_eps};
+            out_probe = d->q_out;
+            break;
+        default: return KX_ERR_BAD_SHAPE;
+    }
+    // 8-byte alignment is what the plain store asks of y; the other outputs are written per element
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, out_probe, 1, K, N, group_size, d->out_kind == KX_OUT_ROW);
+    if (rc != KX_OK) return rc;
+    if (d->in_kind == KX_IN_ATTN && (K % kx::kHeadDim) != 0) return KX_ERR_BAD_SHAPE;
+
+    kx::AwqPlan p = kx::make_valu_plan(1, K, N, long_rows);
+    p.mb = 1;
+    p.mtiles = 1;
+    float* partials = nullptr;
+    uint32_t* counters = nullptr;
+    rc = kx::resolve_workspace(p, 1, N, workspace, workspace_bytes, &partials, &counters);
+    if (rc != KX_OK) return rc;
+    hipStream_t s = kx::as_stream(stream);
+
+#define KX_CHAIN(PRO, EPI) kx::launch_chain<PRO, EPI>(p, fi, rope, res, x, qweight, scales, qzeros, y, partials, counters, K, N, group_size, s)
+#define KX_BY_OUT(PRO)                                                                   \
+    do {                                                                                 \
+        if (d->out_kind == KX_OUT_ROW) KX_CHAIN(PRO, kx::kEpiStore);                     \
+        else if (d->out_kind == KX_OUT_RESIDUAL) KX_CHAIN(PRO, kx::kEpiResidual);        \
+        else KX_CHAIN(PRO, kx::kEpiQkRope);                                              \
+    } while (0)
+    switch (d->in_kind) {
+        case KX_IN_ROW: KX_BY_OUT(kx::kProNone); break;
+        case KX_IN_SWIGLU: KX_BY_OUT(kx::kProSwiGLU); break;
+        case KX_IN_ATTN: KX_BY_OUT(kx::kProAttnMerge); break;
+        default: KX_BY_OUT(kx::kProPreNorm); break;
+    }
+#undef KX_BY_OUT
+#undef KX_CHAIN
     return kx::launch_status();
 }

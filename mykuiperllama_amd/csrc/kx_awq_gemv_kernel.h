@@ -67,6 +67,7 @@ constexpr int kProSwiGLU = 1;   // x[m,k] = bf16( bf16(silu(a[m,k])) * b[m,k] )
 constexpr int kProAddNorm = 2;  // r = bf16(a + b) (b optional), x = gain * bf16(r * rsqrt(mean(r^2) + eps))
 constexpr int kProAddNormLong = 3;  // the same for rows of more than eight elements per thread
 constexpr int kProAttnMerge = 4;  // x = the attention output, merged here from the per-chunk results (M = 1)
+constexpr int kProPreNorm = 5;    // x = gain * bf16(a * rsqrt(mean(a^2) + eps)), the sum of squares given per 256 columns (M = 1)
 constexpr int kNormChunks = 2;  // most 16-byte pieces of a row a thread holds for the sum of squares
 constexpr int kMergeHold = 20;  // per-chunk values a thread holds per element it merges: 80 chunks in four parts
 constexpr int kMergeStatsPerLane = 2;  // chunks per lane of the wave that prepares a head's factors (>= 80 / 64)
@@ -83,6 +84,19 @@ struct FusedInput {
     const float* part_ml;
     int nchunks;
     int heads_per_kv;
+    // kProPreNorm: sum of squares of row `a`, one partial per tile of 256 columns (at most 64)
+    const float* sumsq;
+    int sumsq_parts;
+};
+
+// kEpiResidual: the finished row o is added to the residual stream, out = bf16(in + bf16(o)), and the
+// sum of squares of the new row is left per column tile for the RMSNorm that follows:
+//   sumsq[t] = ((Q0 + Q1) + Q2) + Q3,  Q_i = wave_sum over the 64 columns of quarter i of tile t
+// (kProPreNorm adds the tiles with one more wave_sum, lane = tile).
+struct ResidualTarget {
+    const uint16_t* in;   // bf16 [N]
+    uint16_t* out;        // bf16 [N], may be `in`: a column is read and written by the same thread
+    float* sumsq;         // [ceil(N / 256)]
 };
 
 constexpr float kCodeOffset = 16.0f;
@@ -113,13 +127,14 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 // What happens to the finished sums (EPI below).
 constexpr int kEpiStore = 0;   // y[m, n] = bf16(sum)
 constexpr int kEpiQkRope = 1;  // the row is q | k | v heads of 128: per-head norm, rotation, cache append (M = 1)
+constexpr int kEpiResidual = 2;  // residual add + per-tile sums of squares (M = 1), see ResidualTarget
 
 template <int WAVES, int RT, int MB, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi, RopeTarget rope) {
+    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi, RopeTarget rope, ResidualTarget res) {
     constexpr int SLOTS = WAVES * kSlotsPerWave;
     constexpr int KB = SLOTS * RT;
     constexpr int THREADS = WAVES * kWave;
@@ -127,6 +142,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     constexpr bool NORM = PRO == kProAddNorm || PRO == kProAddNormLong;
     constexpr int NCH = PRO == kProAddNormLong ? kNormChunks : 1;
     constexpr bool MERGE = PRO == kProAttnMerge;
+    constexpr bool PRENORM = PRO == kProPreNorm;
+    static_assert(!PRENORM || MB == 1, "the pre-reduced norm serves one activation row");
     constexpr int HB = KB / kHeadDim > 0 ? KB / kHeadDim : 1;     // heads in the workgroup's K range
     constexpr int EPT = kMergeParts * KB / THREADS;               // (part, row) elements a thread merges
     static_assert(!MERGE || (MB == 1 && KB % kHeadDim == 0 && EPT * THREADS == kMergeParts * KB && HB <= WAVES),
@@ -152,6 +169,19 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const int wcg = ct * kWC + wc;  // word column in the matrix
     const int k0 = kt * KB + slot * RT;
     const bool active = (wcg < nw) && (k0 < K);
+
+    // Small operands of the epilogue and of the pre-reduced norm are requested first of all, so
+    // that they have long arrived when they are needed (clamped addresses, masked use).
+    uint16_t resid_pre = 0;
+    if constexpr (EPI == kEpiResidual) {
+        const int col = ct * kTileCols + tid % kTileCols;
+        resid_pre = res.in[col < N ? col : N - 1];
+    }
+    float tile_ss = 0.0f;
+    if constexpr (PRO == kProPreNorm) {
+        const int part = tid % kWave;
+        tile_ss = fi.sumsq[part < fi.sumsq_parts ? part : fi.sumsq_parts - 1];
+    }
 
     float acc[MB][8];
 #pragma unroll
@@ -209,7 +239,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             own_a[m] = fi.a[at];
             own_b[m] = b_src[at];
         }
-        if constexpr (NORM) own_gain = fi.gain[krow_c];
+        if constexpr (NORM || PRENORM) own_gain = fi.gain[krow_c];
     }
     if constexpr (NORM) {
         const int last_chunk = (K >> 3) - 1;
@@ -300,6 +330,19 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
                 const uint16_t xv = f32_to_bf16(act * bf16_to_f32(own_b[m]));
                 s_x[m][tid] = (stager && m0 + m < M) ? xv : static_cast<uint16_t>(0);
             }
+        }
+        lds_barrier();
+    }
+    if constexpr (PRENORM) {
+        if (tid < kWave) {
+            const float total = wave_sum(tid < fi.sumsq_parts ? tile_ss : 0.0f);
+            if (tid == 0) s_ss[0][0] = 1.0f / sqrtf(total / static_cast<float>(K) + fi.eps);
+        }
+        lds_barrier();
+        if (tid < KB) {
+            const float inv = s_ss[0][0];
+            const float h = bf16_to_f32(own_gain) * bf16_to_f32(f32_to_bf16(bf16_to_f32(own_a[0]) * inv));
+            s_x[0][tid] = stager ? f32_to_bf16(h) : static_cast<uint16_t>(0);
         }
         lds_barrier();
     }
@@ -437,6 +480,28 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     if constexpr (EPI == kEpiStore) {
         splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
                                   &s_prev);
+    } else if constexpr (EPI == kEpiResidual) {
+        static_assert(MB == 1, "the residual epilogue serves one activation row");
+        float sum[MB];
+        if (!splitk_exchange_sum<MB>(psum, sum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials,
+                                     counters, &s_prev)) {
+            return;
+        }
+        __shared__ float s_quarter[kTileCols / kWave];
+        const int col = ct * kTileCols + tid;
+        float r = 0.0f;
+        if (tid < kTileCols && col < N) {
+            const float o = bf16_to_f32(f32_to_bf16(sum[0]));  // the projection's output is a bf16 tensor
+            const uint16_t rbits = f32_to_bf16(bf16_to_f32(resid_pre) + o);
+            res.out[col] = rbits;
+            r = bf16_to_f32(rbits);
+        }
+        if (tid < kTileCols) {
+            const float q = wave_sum(r * r);
+            if (lane == 0) s_quarter[tid / kWave] = q;
+        }
+        __syncthreads();
+        if (tid == 0) res.sumsq[ct] = ((s_quarter[0] + s_quarter[1]) + s_quarter[2]) + s_quarter[3];
     } else {
         static_assert(MB == 1, "the rotary epilogue serves one activation row");
         float sum[MB];
@@ -463,13 +528,13 @@ inline void launch_awq_gemv(const uint16_t* x, const int32_t* qweight, const uin
                             const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
                             int M, int K, int N, int group, int coltiles, int ktiles, int mtiles,
                             hipStream_t stream, const FusedInput& fi = FusedInput{},
-                            const RopeTarget& rope = RopeTarget{}) {
+                            const RopeTarget& rope = RopeTarget{}, const ResidualTarget& res = ResidualTarget{}) {
     dim3 grid(coltiles * ktiles, mtiles, 1);
     dim3 block(WAVES * kWave, 1, 1);
     hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB, PRO, EPI>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group, coltiles, ktiles, fi, rope);
+                       group, coltiles, ktiles, fi, rope, res);
 }
 
 }  // namespace kx

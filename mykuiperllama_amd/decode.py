@@ -112,6 +112,7 @@ class DecodeModel:
         self.act = buf(c.intermediate)
         self.down = buf(c.hidden)
         self.logits = buf(c.vocab)
+        self.ssq = torch.zeros(((c.hidden + 255) // 256,), dtype=torch.float32, device="cuda")
         self.token = torch.zeros(1, dtype=torch.int32, device="cuda")
         self.pos = torch.zeros(1, dtype=torch.int32, device="cuda")
         self.next_token = torch.zeros(1, dtype=torch.int32, device="cuda")
@@ -137,8 +138,19 @@ class DecodeModel:
         capi.gemv_awq_bf16(x, w[0], w[1], w[2], y, self.cfg.group, self.gemv_ws)
 
     def step(self, with_lm_head=True, fused=True):
-        """Enqueue one decode step on torch's current stream (no synchronisation)."""
-        if fused:
+        """Enqueue one decode step on torch's current stream (no synchronisation).
+
+        fused=False       every operator a launch of its own (ten per layer)
+        fused="prologue"  the small operators inside the GEMV launches, arithmetic unchanged: bit for bit
+                          the result of fused=False
+        fused=True        ("chain") additionally the residual add and the sum of squares of the RMSNorm
+                          leave with the epilogue of the producing GEMV, which saves every workgroup of the
+                          consuming GEMV a pass over the whole row; the sum is added in another order, so
+                          results agree with the other two modes to rounding, not bit for bit
+        """
+        if fused is True or fused == "chain":
+            return self._step_chain(with_lm_head)
+        if fused == "prologue":
             return self._step_fused(with_lm_head)
         c = self.cfg
         capi.embedding_bf16(self.embed, self.token, self.x)
@@ -188,6 +200,52 @@ class DecodeModel:
             capi.gemv_awq_swiglu_bf16(self.gu[:, : c.intermediate], self.gu[:, c.intermediate:], qw, sc, qz,
                                       self.down, g, ws)
         capi.add_rmsnorm_bf16(xa, self.down, self.final_norm, self.h, c.eps)
+        if with_lm_head:
+            capi.gemv_bf16(self.h, self.lm_head, self.logits)
+            capi.argmax_bf16(self.logits, self.next_token)
+
+    def _step_chain(self, with_lm_head):
+        c = self.cfg
+        g, ws = c.group, self.gemv_ws
+        H, I = c.hidden, c.intermediate
+        merge_in_o = self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS
+        capi.embedding_bf16(self.embed, self.token, self.x)
+        x, ssq = self.x, self.ssq
+        rope = {"out_kind": capi.OUT_QKV_ROPE, "q_out": self.q, "pos": self.pos, "rope_n_q_heads": c.n_q,
+                "rope_n_kv_heads": c.n_kv, "rope_theta": c.rope_theta, "qk_eps": c.eps}
+        into_residual = {"out_kind": capi.OUT_RESIDUAL, "residual_in": x, "residual_out": x, "sumsq_out": ssq}
+        for li, L in enumerate(self.layers):
+            qw, sc, qz = L["qkv"]
+            if li == 0:  # the embedding row comes without its sums of squares
+                capi.gemv_awq_qkv_rope_bf16(x, None, L["in_norm"], c.eps, None, qw, sc, qz, L["q_norm"], L["k_norm"],
+                                            self.q, self.k_cache[li], self.v_cache[li], c.n_q, c.n_kv, self.pos,
+                                            c.rope_theta, c.eps, g, ws)
+            else:
+                capi.gemv_awq_chain_bf16(dict(rope, in_kind=capi.IN_NORM, norm_row=x, norm_sumsq=ssq,
+                                              norm_parts=ssq.numel(), norm_gain=L["in_norm"], norm_eps=c.eps,
+                                              q_gain=L["q_norm"], k_gain=L["k_norm"], k_cache=self.k_cache[li],
+                                              v_cache=self.v_cache[li]), qw, sc, qz, H, c.qkv_out, g, ws)
+            qw, sc, qz = L["o"]
+            if merge_in_o:
+                capi.attn_decode_partial_bf16(self.q, self.k_cache[li], self.v_cache[li], c.n_q, c.n_kv, self.pos,
+                                              self.max_positions, self.attn_ws)
+                capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_ATTN, attn_workspace=self.attn_ws,
+                                              attn_workspace_bytes=self.attn_ws.numel(), n_q_heads=c.n_q,
+                                              n_kv_heads=c.n_kv, max_positions=self.max_positions),
+                                         qw, sc, qz, c.n_q * c.head_dim, H, g, ws)
+            else:
+                capi.attn_decode_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv,
+                                      self.pos, self.max_positions, self.attn_ws)
+                capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_ROW, x=self.attn),
+                                         qw, sc, qz, c.n_q * c.head_dim, H, g, ws)
+            qw, sc, qz = L["gateup"]
+            capi.gemv_awq_chain_bf16({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": ssq,
+                                      "norm_parts": ssq.numel(), "norm_gain": L["post_norm"], "norm_eps": c.eps,
+                                      "out_kind": capi.OUT_ROW, "y": self.gu}, qw, sc, qz, H, 2 * I, g, ws)
+            qw, sc, qz = L["down"]
+            capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_SWIGLU, gate=self.gu[:, :I],
+                                          up=self.gu[:, I:]), qw, sc, qz, I, H, g, ws)
+        capi.rmsnorm_bf16(x, self.final_norm, self.h, c.eps)
         if with_lm_head:
             capi.gemv_bf16(self.h, self.lm_head, self.logits)
             capi.argmax_bf16(self.logits, self.next_token)

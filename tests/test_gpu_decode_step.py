@@ -125,7 +125,7 @@ class Reference:
         return x, logits
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, "prologue", False])
 def test_decode_steps_match_the_fp32_reference(torch, oracle, fused):
     from mykuiperllama_amd import decode
     cfg = decode.ModelConfig(**CFG)
@@ -167,7 +167,7 @@ def test_fused_and_separate_launches_give_the_same_step(torch):
     model = decode.DecodeModel(cfg, MAXPOS)
     model.prefill_cache_random(CTX)
     results = []
-    for fused in (False, True):
+    for fused in (False, "prologue"):
         model.set_input(9, CTX)
         model.step(fused=fused)
         torch.cuda.synchronize()
@@ -176,7 +176,26 @@ def test_fused_and_separate_launches_give_the_same_step(torch):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
-@pytest.mark.parametrize("fused", [True, False])
+def test_chained_step_agrees_with_the_prologue_step_to_rounding(torch):
+    """The chained launches add the RMSNorm's sum of squares tile by tile: same step up to that rounding."""
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    model = decode.DecodeModel(cfg, MAXPOS)
+    model.prefill_cache_random(CTX)
+    results = []
+    for fused in ("prologue", "chain"):
+        model.set_input(9, CTX)
+        model.step(fused=fused)
+        torch.cuda.synchronize()
+        results.append((model.logits.float().clone(), model.x.float().clone(), model.k_cache[-1][CTX].float().clone()))
+    (la, xa, ka), (lb, xb, kb) = results
+    assert torch.isfinite(lb).all()
+    assert ((la - lb).norm() / la.norm()).item() <= 5e-3
+    assert ((xa - xb).norm() / xa.norm()).item() <= 5e-3
+    assert (ka - kb).abs().max().item() <= 0.05
+
+
+@pytest.mark.parametrize("fused", [True, "prologue", False])
 def test_step_is_capturable_in_a_graph_and_replays_identically(torch, fused):
     """A captured step replayed with the same inputs gives bitwise the same logits as eager."""
     from mykuiperllama_amd import decode
