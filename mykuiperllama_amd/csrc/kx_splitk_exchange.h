@@ -64,22 +64,37 @@ __device__ __forceinline__ bool splitk_exchange_sum(const float (&psum)[ROWS], f
     if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return false;
 
     // Last to arrive: every other workgroup's partials were acknowledged before its increment.
-    // Up to 64 loads are in flight per thread (TB K-tiles of every row at a time); per row the
-    // additions keep the order t = 0, 1, 2, ...
+    // The read-back is a round trip to memory (~1 us, the longest leg of the exchange), so as many
+    // loads as the registers allow go out together: TB K-tiles of every row per thread.  Per row the
+    // additions keep a fixed order: t = 0, 1, 2, ... or, with helpers, the even tiles in that order,
+    // the odd ones likewise, then even + odd.
 #pragma unroll
     for (int r = 0; r < ROWS; r++) sum[r] = 0.0f;
-    if (col_ok) {
-        constexpr int TB = ROWS >= 16 ? 4 : 16;
-        const float* pp = partials + col;
-        for (int t0 = 0; t0 < ktiles; t0 += TB) {
+    constexpr int TB = ROWS >= 16 ? 4 : 16;
+    // One activation row, more K tiles than one batch, and threads to spare: the upper half of a
+    // 512-thread workgroup reads the odd tiles, which halves the number of dependent batches.
+    const bool helpers = ROWS == 1 && ktiles > TB && blockDim.x >= 2 * kTileCols;
+    const int lane_col = tid % kTileCols;
+    // 0: the column's owner, 1: its helper; the same for a whole wave, and said so to the compiler,
+    // which then keeps the K-tile offsets in scalar registers (one vector register of addresses
+    // instead of two per load in flight)
+    const int half = __builtin_amdgcn_readfirstlane(tid / kTileCols);
+    const unsigned hcol = static_cast<unsigned>(ct * kTileCols + lane_col);
+    const int step = helpers ? 2 : 1;
+    if ((helpers ? half < 2 : tid < kTileCols) && hcol < static_cast<unsigned>(N)) {
+        for (int t0 = helpers ? half : 0; t0 < ktiles; t0 += TB * step) {
             float v[ROWS][TB];
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
 #pragma unroll
                 for (int u = 0; u < TB; u++) {
-                    v[r][u] = (m0 + r < M && t0 + u < ktiles)
-                        ? load_agent(pp + static_cast<size_t>(t0 + u) * tstride + static_cast<size_t>(m0 + r) * N)
-                        : 0.0f;
+                    // clamped address, masked value: the loads of a batch are straight-line code
+                    const int t = t0 + u * step;
+                    const int tc = t < ktiles ? t : ktiles - 1;
+                    const int mc = m0 + r < M ? m0 + r : M - 1;
+                    const float* row = partials + static_cast<size_t>(tc) * tstride + static_cast<size_t>(mc) * N;
+                    const float got = load_agent(row + hcol);
+                    v[r][u] = (m0 + r < M && t < ktiles) ? got : 0.0f;
                 }
             }
 #pragma unroll
@@ -88,6 +103,12 @@ __device__ __forceinline__ bool splitk_exchange_sum(const float (&psum)[ROWS], f
                 for (int u = 0; u < TB; u++) sum[r] += v[r][u];
             }
         }
+    }
+    if (helpers) {
+        __shared__ float s_help[kTileCols];
+        if (half == 1) s_help[lane_col] = sum[0];
+        __syncthreads();
+        if (half == 0) sum[0] += s_help[lane_col];
     }
     if (tid == 0) {
         // leave the workspace ready for the next launch
