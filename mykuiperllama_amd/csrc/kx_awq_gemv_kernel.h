@@ -277,9 +277,10 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             for (int m = 0; m < MB; m++) {
 #pragma unroll
                 for (int r8 = 0; r8 < RT / 8; r8++) {
-                    xraw[m][r8] = (m0 + m < M)
-                        ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + m) * K + k0 + 8 * r8)
-                        : make_uint4(0u, 0u, 0u, 0u);
+                    // rows past M read row M - 1 and are zeroed: no branch between the loads
+                    const int mrow = m0 + m < M ? m0 + m : M - 1;
+                    const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(mrow) * K + k0 + 8 * r8);
+                    xraw[m][r8] = (m == 0 || m0 + m < M) ? got : make_uint4(0u, 0u, 0u, 0u);
                 }
             }
         }

@@ -311,7 +311,9 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
 #pragma unroll
         for (int u = 0; u < kMergeBatch; u++) {
             const int c = c0 + u * kMergeParts;
-            v[u] = (c < nchunks && s_factor[c] > 0.0f) ? po[c * cstride] : 0.0f;
+            // straight-line loads: a chunk past the end reads the last one, an empty chunk whatever its
+            // slot holds; attn_merge_step and the guard below leave both out of the sum
+            v[u] = po[(c < nchunks ? c : nchunks - 1) * cstride];
         }
 #pragma unroll
         for (int u = 0; u < kMergeBatch; u++) {
