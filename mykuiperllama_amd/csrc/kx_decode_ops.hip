@@ -152,6 +152,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // the position has arrived.  The chunk then costs one memory round trip.
     const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
     constexpr int ITERS = kAttnChunk / 16;
+    // The G query heads, this lane's eight dims of each, are requested first: loads return in order,
+    // and the scores need q and K but not V, so q must not queue behind the V rows.
+    uint4 qraw[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        qraw[g] = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub);
+    }
     u32x4 kraw[ITERS], vraw[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; it++) {
@@ -167,25 +174,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         vraw[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
             v_cache + pc * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub));
     }
-    // the G query heads, this lane's eight dims of each
-    float qv[G][8];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        unpack8(*reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub), qv[g]);
-    }
     const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
     __builtin_amdgcn_sched_barrier(0);
+    float qv[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) unpack8(qraw[g], qv[g]);
 
     float* out_base = part_out + (static_cast<size_t>(kvh) * nchunks + chunk) * G * kHeadDim;
     float* ml_base = part_ml + (static_cast<size_t>(kvh) * nchunks + chunk) * G * 2;
-    if (p0 >= ctx) {
-        // a chunk past the end of the context contributes nothing: max = -inf, sum = 0
-        if (tid < G) {
-            ml_base[2 * tid] = -INFINITY;
-            ml_base[2 * tid + 1] = 0.0f;
-        }
-        return;
-    }
+    // No early exit for a chunk past the end of the context: a branch on *pos ahead of the loads
+    // lets the compiler sink every K and V load below it, and the chunk then costs the round trip
+    // for *pos and the round trip for the rows one after the other.  Such a chunk runs through with
+    // everything masked and reports max = -inf, sum = 0.
 
     // pass 1: scores
 #pragma unroll
@@ -216,10 +216,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
             m = fmaxf(m, sc[u]);
         }
         m = wave_max(m);
+        const float shift = m == -INFINITY ? 0.0f : m;  // a chunk with no valid position: all weights 0
         float l = 0.0f;
 #pragma unroll
         for (int u = 0; u < PER_LANE; u++) {
-            sc[u] = expf(sc[u] - m);
+            sc[u] = expf(sc[u] - shift);
             l += sc[u];
             s_score[g][lane + u * kWave] = sc[u];
         }
