@@ -1,0 +1,32 @@
+// MultiHeadAttention: grouped-query attention of one query position against cache rows 0 .. pos
+// (the LayerMHA slot, kuiper/include/op/layer.h:15; the reference's mha.h is an empty namespace).
+// out[h, :] = softmax(q[h, :] . K[:, h / G, :] / sqrt(128)) V[:, h / G, :], G = n_q / n_kv in {1, 2, 4, 8}.
+//   input 0    q bf16 [n_q * 128]
+//   input 1    pos int32 [1] on the layer's device
+//   input 2    k_cache bf16 [max_positions, n_kv, 128]     input 3   v_cache, same shape
+//   output 0   bf16 [n_q * 128]
+// A GPU layer owns the workspace of the split over the context (allocated on first use for the
+// cache's max_positions, at most 32768).
+#ifndef KUIPER_INCLUDE_OP_MHA_H
+#define KUIPER_INCLUDE_OP_MHA_H
+
+#include "op/typed_layer.h"
+
+namespace op {
+
+class MultiHeadAttention : public TypedLayer {
+public:
+    explicit MultiHeadAttention(base::DeviceType device_type, int32_t n_q_heads, int32_t n_kv_heads);
+    base::Status check() const override;
+    base::Status forward() override;
+    using TypedLayer::forward;
+
+private:
+    int32_t n_q_ = 0;
+    int32_t n_kv_ = 0;
+    tensor::Tensor workspace_;  // GPU only
+};
+
+}  // namespace op
+
+#endif  // KUIPER_INCLUDE_OP_MHA_H

@@ -1,29 +1,13 @@
 // Host matmul kernels (explicit DeviceCPU layers only).
 #include "matmul_kernel.h"
 
+#include "bf16.h"
+
 #include <cstring>
 #include <vector>
 
 namespace kernel {
 namespace {
-
-inline float bf16_to_float(uint16_t h) {
-    uint32_t u = static_cast<uint32_t>(h) << 16;
-    float f;
-    std::memcpy(&f, &u, sizeof(f));
-    return f;
-}
-
-// round to nearest even; NaN stays quiet NaN
-inline uint16_t float_to_bf16(float f) {
-    uint32_t u;
-    std::memcpy(&u, &f, sizeof(u));
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        return static_cast<uint16_t>((u >> 16) | 0x0040u);
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
-}
 
 inline float half_to_float(uint16_t h) {
     const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
