@@ -27,14 +27,18 @@ inline int kernel_override() {
     return g_kernel_policy;
 }
 
+constexpr int kComputeUnits = 256;  // MI355X
+
 inline bool is_pow2(int v) {
     return v > 0 && (v & (v - 1)) == 0;
 }
 
 // MFMA kernel: four waves per workgroup, each walking `ks` consecutive 32-row steps that must lie in
 // one quantisation group.  Measured on the Qwen3-8B shapes: two steps per wave (256 rows per
-// workgroup) are best for M = 2..4, four steps (512 rows, half the partial sums to exchange) from
-// M = 5 on, where the exchange grows with M.
+// workgroup) are best for M = 2 and for matrices with few column tiles; four steps (512 rows, half
+// the partial sums to exchange) from M = 3 on, where the exchange grows with M (gate 4096 -> 12288
+// at M = 4: 14.9 -> 13.3 us, down 12288 -> 4096: 17.3 -> 14.2 us; q 4096 -> 4096 would be left with
+// 128 workgroups and goes 8.3 -> 10.3 us).
 inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     AwqPlan p;
     p.mfma = true;
@@ -42,7 +46,9 @@ inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     p.mb = M;
     p.mtiles = 1;
     p.waves = 4;
-    int ks = M >= 5 ? 4 : 2;
+    // four steps per wave only where that still leaves a workgroup for every compute unit
+    const bool enough_blocks = static_cast<long>(p.coltiles) * (K / (4 * 4 * kStepRows)) >= kComputeUnits;
+    int ks = (M >= 3 && enough_blocks) ? 4 : 2;
     while (ks > 1 && ks * kStepRows > group) ks /= 2;
     while (ks > 1 && p.waves * ks * kStepRows > K) ks /= 2;
     p.rt = ks;  // steps per wave
@@ -226,7 +232,8 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
         if (M == 1) kx::launch_awq_gemv_mfma<4, KS, 1, 1>(KX_MARGS);            \
         else if (M == 2) kx::launch_awq_gemv_mfma<4, KS, 2, 1>(KX_MARGS);       \
         else if (M <= 4) kx::launch_awq_gemv_mfma<4, KS, 4, 1>(KX_MARGS);       \
-        else kx::launch_awq_gemv_mfma<4, KS, 4, 4>(KX_MARGS);                   \
+        else if (M <= 8) kx::launch_awq_gemv_mfma<4, KS, 8, 1>(KX_MARGS);       \
+        else kx::launch_awq_gemv_mfma<4, KS, 8, 2>(KX_MARGS);                   \
     } while (0)
         if (p.rt == 4) KX_MFMA_BY_M(4);
         else if (p.rt == 2) KX_MFMA_BY_M(2);

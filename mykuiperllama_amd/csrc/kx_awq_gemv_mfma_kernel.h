@@ -62,7 +62,7 @@ __device__ __forceinline__ uint32_t code_pair_to_bf16(uint32_t v, uint32_t magic
 }
 
 // KS: consecutive 32-row steps per wave (they must share a quantisation group);
-// MC: activation rows a workgroup reduces per LDS round (1, 2 or 4); ROUNDS: 1 for M <= 4, else 4.
+// MC: activation rows a workgroup reduces per LDS round (1, 2, 4 or 8); ROUNDS: 2 for M > 8, else 1.
 template <int WAVES, int KS, int MC, int ROUNDS>
 __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
@@ -185,27 +185,36 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
     }
 
     // ---- waves meet in LDS; thread t < 256 then owns tile column t ----
+    // A round carries MC activation rows; a lane holds D rows 4b .. 4b+3 and joins the round they fall in.
+    constexpr int VR = MC < 4 ? MC : 4;  // rows of the lane's four that exist at all
     float psum[ROWS];
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; rd++) {
         if (rd > 0) __syncthreads();  // the previous round has been read
-        if (b == rd) {
-            // D rows 4b + v are activation rows 4*rd + v; the lane's sixteen columns are 16c .. 16c+15
+        const int local0 = 4 * b - rd * MC;  // the lane's first row inside this round
+        if (local0 >= 0 && local0 < MC) {
+            // the lane's sixteen columns are 16c .. 16c+15
 #pragma unroll
-            for (int v = 0; v < MC; v++) {
+            for (int v = 0; v < VR; v++) {
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    f32x4* dst = reinterpret_cast<f32x4*>(&red[wave][v][16 * c + 8 * h]);
+                    f32x4* dst = reinterpret_cast<f32x4*>(&red[wave][local0 + v][16 * c + 8 * h]);
                     dst[0] = f32x4{acc[h][nibble_of(0)][v], acc[h][nibble_of(1)][v], acc[h][nibble_of(2)][v],
                                    acc[h][nibble_of(3)][v]};
                     dst[1] = f32x4{acc[h][nibble_of(4)][v], acc[h][nibble_of(5)][v], acc[h][nibble_of(6)][v],
                                    acc[h][nibble_of(7)][v]};
                 }
-                if (c == 0) xs_red[wave][v] = xs[v];
+                if (c == 0) xs_red[wave][local0 + v] = xs[v];
             }
         }
         __syncthreads();
         if (tid < kTileCols) {
+            float sc[WAVES], zc[WAVES];
+#pragma unroll
+            for (int wv = 0; wv < WAVES; wv++) {
+                sc[wv] = f16_bits_to_f32(s_bits[wv]);
+                zc[wv] = -(128.0f + static_cast<float>((z_word[wv] >> (4 * nibble_of(own_col & 7))) & 0xFu));
+            }
             float qv[MC][WAVES], xv[MC][WAVES];
 #pragma unroll
             for (int v = 0; v < MC; v++) {
@@ -220,16 +229,19 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
                 float total = 0.0f;
 #pragma unroll
                 for (int wv = 0; wv < WAVES; wv++) {
-                    const float s = f16_bits_to_f32(s_bits[wv]);
-                    const float z = static_cast<float>((z_word[wv] >> (4 * nibble_of(own_col & 7))) & 0xFu);
-                    total += s * __builtin_fmaf(-(128.0f + z), xv[v][wv], qv[v][wv]);
+                    total += sc[wv] * __builtin_fmaf(zc[wv], xv[v][wv], qv[v][wv]);
                 }
                 psum[rd * MC + v] = total;
             }
         }
     }
 
-    splitk_exchange_store<ROWS>(psum, 0, M, N, ct, kt, ktiles, ct, partials, counters, y, &s_prev);
+    if constexpr (ROWS >= 8) {
+        static_assert(WAVES * kWave == kTileCols, "the wide exchange is laid out for 256 threads");
+        splitk_exchange_store_wide<ROWS>(psum, M, N, ct, kt, ktiles, partials, counters, y, &s_prev);
+    } else {
+        splitk_exchange_store<ROWS>(psum, 0, M, N, ct, kt, ktiles, ct, partials, counters, y, &s_prev);
+    }
 }
 
 template <int WAVES, int KS, int MC, int ROUNDS>

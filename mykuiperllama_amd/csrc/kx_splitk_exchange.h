@@ -137,6 +137,96 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
     }
 }
 
+// The exchange with the plain epilogue for many activation rows (ROWS = 8 or 16) and a workgroup of
+// exactly 256 threads.  Partial sums go out as above, one column per thread.  The last workgroup
+// reads them back two columns per load: threads 0..127 take rows 0 .. ROWS/2-1 of column pairs
+// 0..127, threads 128..255 the other rows, so a K tile costs a thread ROWS/2 eight-byte loads
+// instead of ROWS four-byte ones and every K tile of the usual shapes is in flight at once.
+// Per output the additions run t = 0, 1, 2, ... as in the narrow exchange.
+template <int ROWS>
+__device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[ROWS], int M, int N, int ct, int kt,
+                                                           int ktiles, float* __restrict__ partials,
+                                                           uint32_t* __restrict__ counters,
+                                                           uint16_t* __restrict__ y, uint32_t* s_prev) {
+    static_assert(ROWS == 8 || ROWS == 16, "row counts the wide read-back is laid out for");
+    const int tid = threadIdx.x;
+    const int col = ct * kTileCols + tid;
+    const bool col_ok = col < N;
+    if (ktiles == 1) {
+        if (col_ok) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (r < M) y[static_cast<size_t>(r) * N + col] = f32_to_bf16(psum[r]);
+            }
+        }
+        return;
+    }
+
+    const size_t tstride = static_cast<size_t>(M) * N;
+    if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            if (r < M) store_agent(partials + static_cast<size_t>(kt) * tstride + static_cast<size_t>(r) * N + col, psum[r]);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    uint32_t* counter = counters + static_cast<size_t>(ct) * kCounterStride;
+    if (tid == 0) {
+        *s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return;
+
+    constexpr int HALF = ROWS / 2;   // rows per thread
+    constexpr int TB = 64 / HALF;    // K tiles per batch: 64 loads in flight
+    const int row0 = __builtin_amdgcn_readfirstlane(tid / (kTileCols / 2)) * HALF;  // the same for a whole wave
+    const unsigned col2 = static_cast<unsigned>(ct * kTileCols + 2 * (tid % (kTileCols / 2)));
+    if (col2 < static_cast<unsigned>(N)) {  // N is even: a pair is all in or all out
+        float lo[HALF], hi[HALF];
+#pragma unroll
+        for (int i = 0; i < HALF; i++) lo[i] = hi[i] = 0.0f;
+        for (int t0 = 0; t0 < ktiles; t0 += TB) {
+            uint64_t v[HALF][TB];
+#pragma unroll
+            for (int i = 0; i < HALF; i++) {
+#pragma unroll
+                for (int u = 0; u < TB; u++) {
+                    // clamped address, masked value: the loads of a batch are straight-line code
+                    const int t = t0 + u;
+                    const int tc = t < ktiles ? t : ktiles - 1;
+                    const int m = row0 + i;
+                    const int mc = m < M ? m : M - 1;
+                    const float* src = partials + static_cast<size_t>(tc) * tstride + static_cast<size_t>(mc) * N + col2;
+                    const uint64_t got = __hip_atomic_load(reinterpret_cast<const uint64_t*>(src), __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT);
+                    v[i][u] = (m < M && t < ktiles) ? got : 0ull;  // all-zero bits are two +0.0f
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < HALF; i++) {
+#pragma unroll
+                for (int u = 0; u < TB; u++) {
+                    lo[i] += __builtin_bit_cast(float, static_cast<uint32_t>(v[i][u]));
+                    hi[i] += __builtin_bit_cast(float, static_cast<uint32_t>(v[i][u] >> 32));
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < HALF; i++) {
+            const int m = row0 + i;
+            if (m < M) {
+                *reinterpret_cast<uint32_t*>(y + static_cast<size_t>(m) * N + col2) = f32x2_to_bf16x2(lo[i], hi[i]);
+            }
+        }
+    }
+    if (tid == 0) {
+        // leave the workspace ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 }  // namespace kx
 
 #endif  // KX_SPLITK_EXCHANGE_H
