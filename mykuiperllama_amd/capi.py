@@ -170,7 +170,7 @@ def gemv_awq_qkv_rope_bf16(residual, delta, gain, eps, residual_out, qweight, sc
 
 
 def set_awq_kernel_policy(policy):
-    """0 = choose by shape, 1 = vector-ALU kernel, 2 = MFMA kernel where the group size allows."""
+    """0 = choose by shape, 1 = vector-ALU kernel, 2 = MFMA kernel where group size and N allow."""
     _check(load().kx_set_awq_kernel_policy(policy))
 
 

@@ -20,14 +20,12 @@ inline int rows_per_block(int waves, int rt) {
     return waves * kSlotsPerWave * rt;
 }
 
-// 0: choose by shape; 1: always the VALU kernel; 2: the MFMA kernel wherever the group size allows
+// 0: choose by shape; 1: always the VALU kernel; 2: the MFMA kernel wherever group size and N allow
 int g_kernel_policy = 0;
 
 inline int kernel_override() {
     return g_kernel_policy;
 }
-
-constexpr int kComputeUnits = 256;  // MI355X
 
 inline bool is_pow2(int v) {
     return v > 0 && (v & (v - 1)) == 0;
@@ -35,10 +33,10 @@ inline bool is_pow2(int v) {
 
 // MFMA kernel: four waves per workgroup, each walking `ks` consecutive 32-row steps that must lie in
 // one quantisation group.  Measured on the Qwen3-8B shapes: two steps per wave (256 rows per
-// workgroup) are best for M = 2 and for matrices with few column tiles; four steps (512 rows, half
-// the partial sums to exchange) from M = 3 on, where the exchange grows with M (gate 4096 -> 12288
-// at M = 4: 14.9 -> 13.3 us, down 12288 -> 4096: 17.3 -> 14.2 us; q 4096 -> 4096 would be left with
-// 128 workgroups and goes 8.3 -> 10.3 us).
+// workgroup) are best up to M = 8, except that long K (down 12288 -> 4096, 48 K tiles) does better
+// with four steps from M = 5 (15.7 -> 14.4 us at M = 8); from M = 9 four steps (512 rows, half the
+// partial sums to exchange) win everywhere (M = 16: q 12.1 -> 10.5, gate 15.6 -> 13.7, down
+// 24.7 -> 18.0 us), even where they leave fewer workgroups than compute units.
 inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     AwqPlan p;
     p.mfma = true;
@@ -46,9 +44,7 @@ inline AwqPlan make_mfma_plan(int M, int K, int N, int group) {
     p.mb = M;
     p.mtiles = 1;
     p.waves = 4;
-    // four steps per wave only where that still leaves a workgroup for every compute unit
-    const bool enough_blocks = static_cast<long>(p.coltiles) * (K / (4 * 4 * kStepRows)) >= kComputeUnits;
-    int ks = (M >= 3 && enough_blocks) ? 4 : 2;
+    int ks = (M >= 9 || (M >= 5 && K >= 8192)) ? 4 : 2;
     while (ks > 1 && ks * kStepRows > group) ks /= 2;
     while (ks > 1 && p.waves * ks * kStepRows > K) ks /= 2;
     p.rt = ks;  // steps per wave
@@ -85,8 +81,9 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true) 
 }
 
 inline AwqPlan make_plan(int M, int K, int N, int group) {
-    // The MFMA kernel needs quantisation groups that tile the workgroup's K range: powers of two.
-    const bool mfma_ok = is_pow2(group);
+    // The MFMA kernel needs quantisation groups that tile the workgroup's K range (powers of two)
+    // and loads two packed words at a time (N a multiple of sixteen).
+    const bool mfma_ok = is_pow2(group) && (N % 16) == 0;
     const int mode = kernel_override();
     const bool mfma = mfma_ok && (mode == 2 || (mode == 0 && M >= 2));
     return mfma ? make_mfma_plan(M, K, N, group) : make_valu_plan(M, K, N);
@@ -167,7 +164,9 @@ inline int resolve_workspace(const AwqPlan& p, int M, int N, void* workspace, si
     if (p.ktiles <= 1) return KX_OK;
     if (!workspace) return KX_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(workspace) % 256) return KX_ERR_ALIGNMENT;
-    const size_t need = kCounterBytes + static_cast<size_t>(p.ktiles) * M * N * sizeof(float);
+    const size_t partial_bytes = static_cast<size_t>(p.ktiles) * M * N * sizeof(float);
+    if (partial_bytes >= (static_cast<size_t>(1) << 32)) return KX_ERR_BAD_SHAPE;  // 32-bit offsets in the read-back
+    const size_t need = kCounterBytes + partial_bytes;
     if (workspace_bytes < need) return KX_ERR_WORKSPACE;
     if (p.coltiles * p.mtiles > kMaxTiles) return KX_ERR_BAD_SHAPE;
     *counters = static_cast<uint32_t*>(workspace);

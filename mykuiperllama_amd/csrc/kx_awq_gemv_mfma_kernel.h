@@ -64,7 +64,7 @@ __device__ __forceinline__ uint32_t code_pair_to_bf16(uint32_t v, uint32_t magic
 // KS: consecutive 32-row steps per wave (they must share a quantisation group);
 // MC: activation rows a workgroup reduces per LDS round (1, 2, 4 or 8); ROUNDS: 2 for M > 8, else 1.
 template <int WAVES, int KS, int MC, int ROUNDS>
-__global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
+__global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
@@ -87,66 +87,55 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
     const int kt = blockIdx.y;
     const int nw = N >> 3;
 
-    const int wcg = ct * 32 + 2 * c;           // first of the lane's two word columns
     const int kwave = kt * KB + wave * WROWS;  // first row of this wave
-    const bool w0_ok = wcg < nw;
-    const bool w1_ok = wcg + 1 < nw;
 
     // ---- loads, all issued before anything is consumed ----
+    // Every load is unconditional: an address that would fall outside is clamped to one inside, and
+    // what it brings is either masked (activations) or lands in outputs that are never stored
+    // (columns past N).  A load under a condition becomes a branch with a full wait behind it, and
+    // a chain of those is a chain of memory round trips.
+    //
     // Scale and zero point of the column this thread will own after the LDS round, one pair per
     // wave of the workgroup (a wave never straddles a quantisation group; waves that share a group
-    // read the same address).  Everything below is indexed at compile time.
+    // read the same address).
     const int own_col = ct * kTileCols + tid;
-    const bool own_ok = (tid < kTileCols) && (own_col < N);
+    const int own_ld = own_col < N ? own_col : N - 1;
     uint16_t s_bits[WAVES];
     uint32_t z_word[WAVES];
 #pragma unroll
     for (int wv = 0; wv < WAVES; wv++) {
         const int krow = kt * KB + wv * WROWS;
-        const bool ok = own_ok && krow < K;
-        const int g = krow >> group_shift;
-        s_bits[wv] = ok ? scales[static_cast<size_t>(g) * N + own_col] : static_cast<uint16_t>(0);
-        z_word[wv] = ok ? qzeros[static_cast<size_t>(g) * nw + (own_col >> 3)] : 0u;
+        const int g = (krow < K ? krow : K - 1) >> group_shift;  // rows past K meet zero activations
+        s_bits[wv] = scales[static_cast<size_t>(g) * N + own_ld];
+        z_word[wv] = qzeros[static_cast<size_t>(g) * nw + (own_ld >> 3)];
     }
+    // The A operand: row c of the activations, whether or not column slot c holds weights.  Rows
+    // past M and steps past K (K is a multiple of 32: a step is all in or all out) are zeros.
     uint4 xa[KS];
-    uint32_t w[KS][8][2];
+    const int x_row = c < M ? c : M - 1;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        xa[ks] = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-        for (int r = 0; r < 8; r++) w[ks][r][0] = w[ks][r][1] = 0u;
+        const int kstep = kwave + ks * kStepRows;
+        const int kld = kstep < K ? kstep : K - kStepRows;
+        const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(x_row) * K + kld + 8 * b);
+        const bool live = c < M && kstep < K;
+        xa[ks] = make_uint4(live ? got.x : 0u, live ? got.y : 0u, live ? got.z : 0u, live ? got.w : 0u);
     }
-    if (c < M) {
-        // the A operand: row c of the activations, whether or not column slot c holds weights
+    // The lane's two word columns, eight rows per step, both words in one load: the host sends only
+    // N that are multiples of sixteen here, so word rows are 8-byte aligned.
+    uint32_t w[KS][8][2];
+    const int wc_first = ct * 32 + 2 * c;
+    const int wc0 = wc_first < nw ? wc_first : nw - 2;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int kstep = kwave + ks * kStepRows;
-            if (kstep < K) xa[ks] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(c) * K + kstep + 8 * b);
-        }
-    }
-    if (w0_ok) {
-        const bool pair_loads = (nw & 1) == 0;  // rows are 8-byte aligned: both words in one load
+    for (int ks = 0; ks < KS; ks++) {
+        const int kstep = kwave + ks * kStepRows;
+        const int k0 = (kstep < K ? kstep : K - kStepRows) + 8 * b;  // first of the lane's eight rows
+        const uint32_t* wp = qweight + static_cast<size_t>(k0) * nw + wc0;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int kstep = kwave + ks * kStepRows;
-            if (kstep < K) {  // K is a multiple of 32: a step is all in or all out (wave-uniform)
-                const int k0 = kstep + 8 * b;  // first of the lane's eight rows
-                const uint32_t* wp = qweight + static_cast<size_t>(k0) * nw + wcg;
-                if (pair_loads) {
-#pragma unroll
-                    for (int r = 0; r < 8; r++) {
-                        const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(wp + static_cast<size_t>(r) * nw));
-                        w[ks][r][0] = v.x;
-                        w[ks][r][1] = v.y;
-                    }
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 8; r++) {
-                        w[ks][r][0] = __builtin_nontemporal_load(wp + static_cast<size_t>(r) * nw);
-                        if (w1_ok) w[ks][r][1] = __builtin_nontemporal_load(wp + static_cast<size_t>(r) * nw + 1);
-                    }
-                }
-            }
+        for (int r = 0; r < 8; r++) {
+            const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(wp + static_cast<size_t>(r) * nw));
+            w[ks][r][0] = v.x;
+            w[ks][r][1] = v.y;
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -182,6 +171,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
                     a_op, as_bf16x8(bop[p][0], bop[p][1], bop[p][2], bop[p][3]), ks == 0 ? zero4 : acc[h][p], 0, 0, 0);
             }
         }
+        // a step is worked through while the loads of the later steps are still in flight
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- waves meet in LDS; thread t < 256 then owns tile column t ----
@@ -236,7 +227,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_mfma_kernel(
         }
     }
 
-    if constexpr (ROWS >= 8) {
+    if constexpr (ROWS >= 4) {
         static_assert(WAVES * kWave == kTileCols, "the wide exchange is laid out for 256 threads");
         splitk_exchange_store_wide<ROWS>(psum, M, N, ct, kt, ktiles, partials, counters, y, &s_prev);
     } else {

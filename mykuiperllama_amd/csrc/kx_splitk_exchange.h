@@ -137,7 +137,7 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
     }
 }
 
-// The exchange with the plain epilogue for many activation rows (ROWS = 8 or 16) and a workgroup of
+// The exchange with the plain epilogue for several activation rows (ROWS = 4, 8 or 16) and a workgroup of
 // exactly 256 threads.  Partial sums go out as above, one column per thread.  The last workgroup
 // reads them back two columns per load: threads 0..127 take rows 0 .. ROWS/2-1 of column pairs
 // 0..127, threads 128..255 the other rows, so a K tile costs a thread ROWS/2 eight-byte loads
@@ -148,7 +148,7 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
                                                            int ktiles, float* __restrict__ partials,
                                                            uint32_t* __restrict__ counters,
                                                            uint16_t* __restrict__ y, uint32_t* s_prev) {
-    static_assert(ROWS == 8 || ROWS == 16, "row counts the wide read-back is laid out for");
+    static_assert(ROWS == 4 || ROWS == 8 || ROWS == 16, "row counts the wide read-back is laid out for");
     const int tid = threadIdx.x;
     const int col = ct * kTileCols + tid;
     const bool col_ok = col < N;
@@ -180,15 +180,26 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
     if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return;
 
     constexpr int HALF = ROWS / 2;   // rows per thread
-    constexpr int TB = 64 / HALF;    // K tiles per batch: 64 loads in flight
+    constexpr int TB = HALF >= 4 ? 64 / HALF : 16;  // K tiles per batch: up to 64 loads in flight
     const int row0 = __builtin_amdgcn_readfirstlane(tid / (kTileCols / 2)) * HALF;  // the same for a whole wave
     const unsigned col2 = static_cast<unsigned>(ct * kTileCols + 2 * (tid % (kTileCols / 2)));
+    // Buffer loads: the lane's column is one 32-bit register shared by every load, the row's offset
+    // (the same in every lane) a scalar register, so a load in flight costs its two data registers
+    // and nothing else.  Cache policy 16 is the device-scope bit (sc1), as on the loads above.
+    // The host keeps the partial sums below 4 GiB.
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        partials, 0, static_cast<int>(static_cast<uint32_t>(static_cast<size_t>(ktiles) * tstride * sizeof(float))),
+        0x00020000);
+    constexpr int kDeviceScope = 16;
     if (col2 < static_cast<unsigned>(N)) {  // N is even: a pair is all in or all out
+        const int lane_bytes = static_cast<int>(col2 * sizeof(float));
         float lo[HALF], hi[HALF];
 #pragma unroll
         for (int i = 0; i < HALF; i++) lo[i] = hi[i] = 0.0f;
         for (int t0 = 0; t0 < ktiles; t0 += TB) {
-            uint64_t v[HALF][TB];
+            // two scalars per load: a bit cast applied to one element of a vector (v.y) reads
+            // element 0 with this compiler
+            uint32_t va[HALF][TB], vb[HALF][TB];
 #pragma unroll
             for (int i = 0; i < HALF; i++) {
 #pragma unroll
@@ -198,18 +209,20 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
                     const int tc = t < ktiles ? t : ktiles - 1;
                     const int m = row0 + i;
                     const int mc = m < M ? m : M - 1;
-                    const float* src = partials + static_cast<size_t>(tc) * tstride + static_cast<size_t>(mc) * N + col2;
-                    const uint64_t got = __hip_atomic_load(reinterpret_cast<const uint64_t*>(src), __ATOMIC_RELAXED,
-                                                           __HIP_MEMORY_SCOPE_AGENT);
-                    v[i][u] = (m < M && t < ktiles) ? got : 0ull;  // all-zero bits are two +0.0f
+                    // M*N and N are multiples of eight: the row starts on an 8-byte boundary
+                    const uint32_t row_pairs = static_cast<uint32_t>((static_cast<size_t>(tc) * tstride + static_cast<size_t>(mc) * N) / 2);
+                    const u32x2 got = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_bytes, static_cast<int>(row_pairs * 8u), kDeviceScope);
+                    const bool live = m < M && t < ktiles;
+                    va[i][u] = live ? got.x : 0u;  // all-zero bits are +0.0f
+                    vb[i][u] = live ? got.y : 0u;
                 }
             }
 #pragma unroll
             for (int i = 0; i < HALF; i++) {
 #pragma unroll
                 for (int u = 0; u < TB; u++) {
-                    lo[i] += __builtin_bit_cast(float, static_cast<uint32_t>(v[i][u]));
-                    hi[i] += __builtin_bit_cast(float, static_cast<uint32_t>(v[i][u] >> 32));
+                    lo[i] += __builtin_bit_cast(float, va[i][u]);
+                    hi[i] += __builtin_bit_cast(float, vb[i][u]);
                 }
             }
         }
