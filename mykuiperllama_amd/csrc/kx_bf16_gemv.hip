@@ -18,7 +18,9 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 }
 
 constexpr int kRowsPerBlock = 4;  // one wave each
-constexpr int kUnroll = 4;        // 16-byte loads in flight per lane
+// 16-byte weight loads in flight per lane: a row of 4096 in one sweep (four measured slower for
+// every M, also where several activation rows compete for the registers)
+constexpr int kUnroll = 8;
 
 template <int MB>
 __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
@@ -26,46 +28,52 @@ __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
     int M, int K, int N, int m0) {
     const int lane = threadIdx.x % kWave;
     const int n = blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-    if (n >= N) return;
+    // A wave past the last row works on the last row again and stores nothing: no wave leaves
+    // early, no load sits under a condition.
+    const int n_ld = n < N ? n : N - 1;
     const int chunks = K >> 3;  // 16-byte pieces per row
-    const u32x4* wrow = reinterpret_cast<const u32x4*>(w + static_cast<size_t>(n) * K);
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(w + static_cast<size_t>(n_ld) * K);
+    const uint4* xrow[MB];
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+        const int mr = m0 + m < M ? m0 + m : M - 1;  // rows past M repeat the last one, never stored
+        xrow[m] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(mr) * K);
+    }
 
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; m++) acc[m] = 0.0f;
 
     for (int c0 = lane; c0 < chunks; c0 += kWave * kUnroll) {
+        // Clamped addresses, masked weights: the loads of a sweep are straight-line code and all
+        // in flight together (a load under a condition becomes a branch with a full wait behind it).
         u32x4 wv[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const int c = c0 + u * kWave;
-            wv[u] = c < chunks ? __builtin_nontemporal_load(wrow + c) : u32x4{0u, 0u, 0u, 0u};
+            wv[u] = __builtin_nontemporal_load(wrow + (c < chunks ? c : chunks - 1));
         }
+        __builtin_amdgcn_sched_barrier(0);  // every weight load is out before the first is waited for
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const int c = c0 + u * kWave;
-            if (c < chunks) {
+            const bool live = c < chunks;
+            const int cl = live ? c : chunks - 1;
+            const uint32_t w0 = live ? wv[u].x : 0u, w1 = live ? wv[u].y : 0u;
+            const uint32_t w2 = live ? wv[u].z : 0u, w3 = live ? wv[u].w : 0u;
 #pragma unroll
-                for (int m = 0; m < MB; m++) {
-                    if (m0 + m < M) {
-                        const uint4 xv = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + m) * K)[c];
-                        acc[m] = dot2_bf16(wv[u].x, xv.x, acc[m]);
-                        acc[m] = dot2_bf16(wv[u].y, xv.y, acc[m]);
-                        acc[m] = dot2_bf16(wv[u].z, xv.z, acc[m]);
-                        acc[m] = dot2_bf16(wv[u].w, xv.w, acc[m]);
-                    }
-                }
+            for (int m = 0; m < MB; m++) {
+                const uint4 xv = xrow[m][cl];
+                acc[m] = dot2_bf16(w0, xv.x, acc[m]);
+                acc[m] = dot2_bf16(w1, xv.y, acc[m]);
+                acc[m] = dot2_bf16(w2, xv.z, acc[m]);
+                acc[m] = dot2_bf16(w3, xv.w, acc[m]);
             }
         }
     }
 #pragma unroll
-    for (int m = 0; m < MB; m++) {
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) {
-            acc[m] += __shfl_xor(acc[m], off, kWave);
-        }
-    }
-    if (lane == 0) {
+    for (int m = 0; m < MB; m++) acc[m] = wave_sum(acc[m]);
+    if (lane == 0 && n < N) {
 #pragma unroll
         for (int m = 0; m < MB; m++) {
             if (m0 + m < M) y[static_cast<size_t>(m0 + m) * N + n] = f32_to_bf16(acc[m]);

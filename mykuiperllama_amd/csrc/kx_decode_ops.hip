@@ -390,22 +390,24 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* 
     };
     const bool wide = (reinterpret_cast<uintptr_t>(x) % 16) == 0;
     const int chunks = wide ? n / 8 : 0;
-    for (int c0 = threadIdx.x; c0 < chunks; c0 += 4 * kArgmaxThreads) {
-        uint4 raw[4];
+    constexpr int kInFlight = 8;  // 16-byte loads per thread and sweep
+    for (int c0 = threadIdx.x; c0 < chunks; c0 += kInFlight * kArgmaxThreads) {
+        // clamped addresses: the loads of a sweep are straight-line code, all in flight together;
+        // a piece past the end is looked at with values and indices that can never win
+        uint4 raw[kInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kInFlight; u++) {
             const int c = c0 + u * kArgmaxThreads;
-            raw[u] = c < chunks ? reinterpret_cast<const uint4*>(x)[c] : make_uint4(0u, 0u, 0u, 0u);
+            raw[u] = reinterpret_cast<const uint4*>(x)[c < chunks ? c : chunks - 1];
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kInFlight; u++) {
             const int c = c0 + u * kArgmaxThreads;
-            if (c < chunks) {
-                float v[8];
-                unpack8(raw[u], v);
+            const bool live = c < chunks;
+            float v[8];
+            unpack8(raw[u], v);
 #pragma unroll
-                for (int i = 0; i < 8; i++) consider(v[i], 8 * c + i);
-            }
+            for (int i = 0; i < 8; i++) consider(live ? v[i] : -INFINITY, live ? 8 * c + i : 0x7fffffff);
         }
     }
     for (int i = 8 * chunks + threadIdx.x; i < n; i += kArgmaxThreads) consider(bf16_to_f32(x[i]), i);

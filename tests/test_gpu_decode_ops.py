@@ -183,3 +183,18 @@ def test_swiglu_add_embedding_argmax(capi, torch):
     capi.argmax_bf16(logits.cuda(), idx)
     torch.cuda.synchronize()
     assert idx.item() == 123
+    # ragged lengths (shorter than one 16-byte piece, not a multiple of eight, the maximum in the
+    # last element) and a pointer off the 16-byte grid
+    g = torch.Generator().manual_seed(5)
+    for n in (1, 7, 8, 9, 1000, 8193, 65537):
+        for shift in (0, 1):
+            buf = torch.randn(n + shift, generator=g).bfloat16()
+            view = buf[shift:]
+            for where in (n - 1, n // 2, 0):
+                vals = view.clone()
+                vals[where] = 60.0
+                dev = torch.empty(n + shift, dtype=torch.bfloat16, device="cuda")
+                dev[shift:] = vals.cuda()
+                capi.argmax_bf16(dev[shift:], idx)
+                torch.cuda.synchronize()
+                assert idx.item() == where, (n, shift, where)
