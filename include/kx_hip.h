@@ -118,7 +118,8 @@ int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t* delta, co
  * the fused q|k|v projection (N = (n_q_heads + 2 n_kv_heads) * 128, query heads first, then key
  * heads, then value heads), and on the finished row what kx_qk_norm_rope_bf16 does: per-head RMSNorm
  * of the query and key heads, rotation at *pos, queries to q_out, keys and values into row *pos of
- * the caches.  Bitwise the result of kx_gemv_awq_addnorm_bf16 followed by kx_qk_norm_rope_bf16.
+ * the caches (which hold cache_positions rows; a position outside them writes no row).
+ * Bitwise the result of kx_gemv_awq_addnorm_bf16 followed by kx_qk_norm_rope_bf16.
  * n_q_heads + 2 n_kv_heads must be even (a column tile of 256 holds whole heads); head_dim = 128.
  * Replaces: LayerAdd + LayerRMSNorm + LayerMatmul + LayerRMSNorm (heads) + LayerRope back to back
  * (slots kuiper/include/op/layer.h:8-20; not implemented in the reference). */
@@ -127,8 +128,8 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
                               const uint16_t* scales, const int32_t* qzeros, const uint16_t* q_gain,
                               const uint16_t* k_gain, uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache,
                               int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
-                              float rope_theta, float qk_eps, int32_t K, int32_t group_size, void* workspace,
-                              size_t workspace_bytes, void* stream);
+                              int32_t cache_positions, float rope_theta, float qk_eps, int32_t K,
+                              int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Chained GEMV (M = 1): one launch whose activations come from the previous operator of a decoder
@@ -149,7 +150,7 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
  *                                                        in place), sumsq_out[t] = sum of squares of columns
  *                                                        256 t .. 256 t + 255 of residual_out, t < ceil(N / 256)
  *   KX_OUT_QKV_ROPE q_gain, k_gain, q_out, k_cache, v_cache, pos, rope_n_q_heads, rope_n_kv_heads,
- *                   rope_theta, qk_eps                   as kx_gemv_awq_qkv_rope_bf16 (N = (n_q + 2 n_kv) * 128)
+ *                   cache_positions, rope_theta, qk_eps  as kx_gemv_awq_qkv_rope_bf16 (N = (n_q + 2 n_kv) * 128)
  *
  * The sum of squares of KX_OUT_RESIDUAL / KX_IN_NORM is added tile by tile, an order of its own:
  * results agree with kx_add_rmsnorm_bf16 followed by the GEMV to within the rounding of that sum
@@ -191,6 +192,7 @@ typedef struct kx_chain_desc {
     float qk_eps;
     int32_t rope_n_q_heads;
     int32_t rope_n_kv_heads;
+    int32_t cache_positions;
     /* KX_OUT_ROW */
     uint16_t* y;
     /* KX_OUT_RESIDUAL */
@@ -247,7 +249,8 @@ int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const in
  *   kx_qk_norm_rope_bf16  qkv = [q heads | k heads | v heads] x 128: RMSNorm over each q / k head with
  *                         its 128-element gain, rotary embedding at *pos (rotate-half convention,
  *                         frequencies theta^(-i/64)), q to q_out, k and v to row *pos of the caches
- *                         (bf16 [max_positions][n_kv_heads][128]).  head_dim must be 128.
+ *                         (bf16 [cache_positions][n_kv_heads][128]; a position outside
+ *                         0 .. cache_positions-1 writes no cache row).  head_dim must be 128.
  *   kx_attn_decode_bf16   GQA attention of one query position against cache rows 0 .. *pos:
  *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv in
  *                         {1,2,4,8}; split over the context in chunks of 64 positions, merged by
@@ -267,7 +270,8 @@ int kx_add_rmsnorm_bf16(uint16_t* x_inout, const uint16_t* delta, const uint16_t
                         int32_t rows, int32_t n, float eps, void* stream);
 int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain, uint16_t* q_out,
                          uint16_t* k_cache, uint16_t* v_cache, int32_t n_q_heads, int32_t n_kv_heads,
-                         int32_t head_dim, const int32_t* pos, float rope_theta, float eps, void* stream);
+                         int32_t head_dim, const int32_t* pos, int32_t cache_positions, float rope_theta, float eps,
+                         void* stream);
 size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head_dim, int32_t max_positions);
 int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, uint16_t* out,
                         int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,

@@ -27,13 +27,13 @@ SIGNATURES = {
     "kx_gemv_awq_addnorm_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I32, _I32,
                                                 _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_qkv_rope_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _P, _P, _P, _P,
-                                                 _I32, _I32, _I32, _P, ctypes.c_float, ctypes.c_float, _I32, _I32,
-                                                 _P, _SZ, _P]),
+                                                 _I32, _I32, _I32, _P, _I32, ctypes.c_float, ctypes.c_float, _I32,
+                                                 _I32, _P, _SZ, _P]),
     "kx_gemv_awq_chain_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_awq_unpack_u8": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "kx_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
     "kx_add_rmsnorm_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, ctypes.c_float, _P]),
-    "kx_qk_norm_rope_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, ctypes.c_float,
+    "kx_qk_norm_rope_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, ctypes.c_float,
                                             ctypes.c_float, _P]),
     "kx_attn_decode_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kx_attn_decode_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _SZ, _P]),
@@ -58,7 +58,7 @@ class ChainDesc(ctypes.Structure):
         ("n_q_heads", _I32), ("n_kv_heads", _I32), ("max_positions", _I32),
         ("norm_parts", _I32), ("norm_row", _P), ("norm_sumsq", _P), ("norm_gain", _P), ("norm_eps", ctypes.c_float),
         ("rope_theta", ctypes.c_float), ("qk_eps", ctypes.c_float),
-        ("rope_n_q_heads", _I32), ("rope_n_kv_heads", _I32),
+        ("rope_n_q_heads", _I32), ("rope_n_kv_heads", _I32), ("cache_positions", _I32),
         ("y", _P),
         ("residual_in", _P), ("residual_out", _P), ("sumsq_out", _P),
         ("q_gain", _P), ("k_gain", _P), ("q_out", _P), ("k_cache", _P), ("v_cache", _P), ("pos", _P),
@@ -160,12 +160,14 @@ def gemv_awq_addnorm_bf16(residual, delta, gain, eps, residual_out, qweight, sca
 
 def gemv_awq_qkv_rope_bf16(residual, delta, gain, eps, residual_out, qweight, scales, qzeros, q_gain, k_gain,
                            q_out, k_cache, v_cache, n_q, n_kv, pos, rope_theta, qk_eps, group_size, workspace):
-    """add + RMSNorm, fused q|k|v projection, per-head norm + rotation + cache append; one row."""
+    """add + RMSNorm, fused q|k|v projection, per-head norm + rotation + cache append; one row.
+    k_cache / v_cache: bf16 [positions, n_kv, 128]; the first dimension is the capacity the kernel guards."""
     K = residual.shape[-1]
     _check(load().kx_gemv_awq_qkv_rope_bf16(_ptr(residual), _ptr(delta), _ptr(gain), eps, _ptr(residual_out),
                                             _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(q_gain), _ptr(k_gain),
                                             _ptr(q_out), _ptr(k_cache), _ptr(v_cache), n_q, n_kv, 128, _ptr(pos),
-                                            rope_theta, qk_eps, K, group_size, _ptr(workspace),
+                                            _cache_positions(k_cache, v_cache), rope_theta, qk_eps, K, group_size,
+                                            _ptr(workspace),
                                             0 if workspace is None else workspace.numel(), _stream()))
 
 
@@ -205,9 +207,17 @@ def add_rmsnorm_bf16(x_inout, delta, gain, y, eps):
                                       eps, _stream()))
 
 
+def _cache_positions(k_cache, v_cache):
+    """Rows of a KV cache pair laid out [positions, n_kv, 128] (the capacity the append is guarded by)."""
+    if k_cache is None or v_cache is None:
+        return 1  # the call fails on the null pointer
+    return min(k_cache.shape[0], v_cache.shape[0])
+
+
 def qk_norm_rope_bf16(qkv, q_gain, k_gain, q_out, k_cache, v_cache, n_q, n_kv, pos, theta, eps):
     _check(load().kx_qk_norm_rope_bf16(_ptr(qkv), _ptr(q_gain), _ptr(k_gain), _ptr(q_out), _ptr(k_cache),
-                                       _ptr(v_cache), n_q, n_kv, 128, _ptr(pos), theta, eps, _stream()))
+                                       _ptr(v_cache), n_q, n_kv, 128, _ptr(pos), _cache_positions(k_cache, v_cache),
+                                       theta, eps, _stream()))
 
 
 def attn_decode_workspace(n_q, max_positions, device="cuda"):
@@ -240,6 +250,8 @@ def gemv_awq_chain_bf16(desc, qweight, scales, qzeros, K, N, group_size, workspa
     """One link of a decoder layer's chain: see kx_chain_desc.  `desc` maps field names to tensors,
     None or scalars; tensors are passed by address."""
     d = ChainDesc()
+    if "cache_positions" not in desc and desc.get("k_cache") is not None and desc.get("v_cache") is not None:
+        d.cache_positions = _cache_positions(desc["k_cache"], desc["v_cache"])
     for name, value in desc.items():
         setattr(d, name, value.data_ptr() if hasattr(value, "data_ptr") else value)
     _check(load().kx_gemv_awq_chain_bf16(ctypes.byref(d), _ptr(qweight), _ptr(scales), _ptr(qzeros), K, N, group_size,

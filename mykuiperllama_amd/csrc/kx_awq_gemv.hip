@@ -322,13 +322,16 @@ extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_
                                          const uint16_t* scales, const int32_t* qzeros, const uint16_t* q_gain,
                                          const uint16_t* k_gain, uint16_t* q_out, uint16_t* k_cache,
                                          uint16_t* v_cache, int32_t n_q_heads, int32_t n_kv_heads,
-                                         int32_t head_dim, const int32_t* pos, float rope_theta, float qk_eps,
+                                         int32_t head_dim, const int32_t* pos, int32_t cache_positions,
+                                         float rope_theta, float qk_eps,
                                          int32_t K, int32_t group_size, void* workspace,
                                          size_t workspace_bytes, void* stream) {
     if (!residual || !gain || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) {
         return KX_ERR_NULL_POINTER;
     }
-    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || !(rope_theta > 1.0f)) return KX_ERR_BAD_SHAPE;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || cache_positions < 1 || !(rope_theta > 1.0f)) {
+        return KX_ERR_BAD_SHAPE;
+    }
     // a column tile of 256 must hold whole heads
     if ((n_q_heads + 2 * n_kv_heads) % (kx::kTileCols / kx::kHeadDim) != 0) return KX_ERR_BAD_SHAPE;
     const int N = (n_q_heads + 2 * n_kv_heads) * kx::kHeadDim;
@@ -352,7 +355,7 @@ extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_
     fi.r_out = residual_out;
     fi.ld = K;
     fi.eps = eps;
-    const kx::RopeTarget rope{q_gain, k_gain, q_out, k_cache, v_cache, pos, n_q_heads, n_kv_heads,
+    const kx::RopeTarget rope{q_gain, k_gain, q_out, k_cache, v_cache, pos, cache_positions, n_q_heads, n_kv_heads,
                               log2f(rope_theta), qk_eps};
     if ((K >> 3) <= p.waves * kx::kWave) {
         kx::launch_qkv<kx::kProAddNorm>(p, fi, rope, qweight, scales, qzeros, partials, counters, K, N, group_size,
@@ -509,12 +512,12 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
             break;
         case KX_OUT_QKV_ROPE:
             if (!d->q_gain || !d->k_gain || !d->q_out || !d->k_cache || !d->v_cache || !d->pos) return KX_ERR_NULL_POINTER;
-            if (d->rope_n_q_heads < 1 || d->rope_n_kv_heads < 1 || !(d->rope_theta > 1.0f) ||
+            if (d->rope_n_q_heads < 1 || d->rope_n_kv_heads < 1 || d->cache_positions < 1 || !(d->rope_theta > 1.0f) ||
                 N != (d->rope_n_q_heads + 2 * d->rope_n_kv_heads) * kx::kHeadDim ||
                 (d->rope_n_q_heads + 2 * d->rope_n_kv_heads) % (kx::kTileCols / kx::kHeadDim) != 0) {
                 return KX_ERR_BAD_SHAPE;
             }
-            rope = kx::RopeTarget{d->q_gain, d->k_gain, d->q_out, d->k_cache, d->v_cache, d->pos,
+            rope = kx::RopeTarget{d->q_gain, d->k_gain, d->q_out, d->k_cache, d->v_cache, d->pos, d->cache_positions,
                                   d->rope_n_q_heads, d->rope_n_kv_heads, log2f(d->rope_theta), d->qk_eps};
             out_probe = d->q_out;
             break;

@@ -467,12 +467,15 @@ extern "C" int kx_add_rmsnorm_bf16(uint16_t* x_inout, const uint16_t* delta, con
 
 extern "C" int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain,
                                     uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int32_t n_q_heads,
-                                    int32_t n_kv_heads, int32_t head_dim, const int32_t* pos, float rope_theta,
-                                    float eps, void* stream) {
+                                    int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
+                                    int32_t cache_positions, float rope_theta, float eps, void* stream) {
     if (!qkv || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) return KX_ERR_NULL_POINTER;
-    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || !(rope_theta > 1.0f)) return KX_ERR_BAD_SHAPE;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || cache_positions < 1 || !(rope_theta > 1.0f)) {
+        return KX_ERR_BAD_SHAPE;
+    }
     const int heads = n_q_heads + 2 * n_kv_heads;
-    kx::RopeTarget t{q_gain, k_gain, q_out, k_cache, v_cache, pos, n_q_heads, n_kv_heads, log2f(rope_theta), eps};
+    kx::RopeTarget t{q_gain, k_gain, q_out, k_cache, v_cache, pos, cache_positions, n_q_heads, n_kv_heads,
+                     log2f(rope_theta), eps};
     hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4), dim3(256), 0, kx::as_stream(stream), qkv, t);
     return kx::launch_status();
 }

@@ -16,9 +16,10 @@ struct RopeTarget {
     const uint16_t* q_gain;   // bf16 [128]
     const uint16_t* k_gain;   // bf16 [128]
     uint16_t* q_out;          // bf16 [n_q * 128]
-    uint16_t* k_cache;        // bf16 [max_pos][n_kv][128]; row *pos is written
+    uint16_t* k_cache;        // bf16 [cache_positions][n_kv][128]; row *pos is written
     uint16_t* v_cache;
     const int32_t* pos;       // device scalar
+    int cache_positions;      // rows the caches hold: a position outside 0 .. cache_positions-1 writes no row
     int n_q;
     int n_kv;
     float log2_theta;
@@ -33,10 +34,13 @@ struct RopeTarget {
 __device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bits, int head, int lane,
                                                   const RopeTarget& t) {
     const int pos = t.pos[0];
+    const bool row_ok = static_cast<unsigned>(pos) < static_cast<unsigned>(t.cache_positions);
     if (head >= t.n_q + t.n_kv) {  // value head: straight into the cache
-        uint16_t* dst = t.v_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q - t.n_kv)) * kHeadDim;
-        dst[lane] = a_bits;
-        dst[lane + 64] = b_bits;
+        if (row_ok) {
+            uint16_t* dst = t.v_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q - t.n_kv)) * kHeadDim;
+            dst[lane] = a_bits;
+            dst[lane + 64] = b_bits;
+        }
         return;
     }
     const float a = bf16_to_f32(a_bits);
@@ -57,8 +61,10 @@ __device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bi
     const float ob = xb * c + xa * s;
     uint16_t* dst = is_q ? t.q_out + static_cast<size_t>(head) * kHeadDim
                          : t.k_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q)) * kHeadDim;
-    dst[lane] = f32_to_bf16(oa);
-    dst[lane + 64] = f32_to_bf16(ob);
+    if (is_q || row_ok) {
+        dst[lane] = f32_to_bf16(oa);
+        dst[lane + 64] = f32_to_bf16(ob);
+    }
 }
 
 }  // namespace kx

@@ -78,9 +78,14 @@ void rope_kernel_cu(const tensor::Tensor& qkv, const tensor::Tensor& q_gain, con
     expect_gpu(v_cache);
     CHECK_EQ(qkv.size(), static_cast<size_t>(n_q_heads + 2 * n_kv_heads) * kHeadDim);
     CHECK_EQ(q_out.size(), static_cast<size_t>(n_q_heads) * kHeadDim);
+    // rows of [n_kv_heads][128] the caches hold: the kernel writes no row outside them
+    const size_t row = static_cast<size_t>(n_kv_heads) * kHeadDim;
+    CHECK_EQ(k_cache.size(), v_cache.size());
+    CHECK(k_cache.size() >= row && k_cache.size() % row == 0) << "KV cache is not [positions][n_kv_heads][128]";
+    const int32_t cache_positions = static_cast<int32_t>(k_cache.size() / row);
     const int rc = kx_qk_norm_rope_bf16(qkv.ptr<uint16_t>(), q_gain.ptr<uint16_t>(), k_gain.ptr<uint16_t>(),
                                         out_ptr(q_out), out_ptr(k_cache), out_ptr(v_cache), n_q_heads, n_kv_heads,
-                                        kHeadDim, pos.ptr<int32_t>(), theta, eps, stream);
+                                        kHeadDim, pos.ptr<int32_t>(), cache_positions, theta, eps, stream);
     CHECK(rc == KX_OK) << "RoPE kernel launch failed: " << kx_error_string(rc);
 }
 

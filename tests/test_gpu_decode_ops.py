@@ -120,6 +120,24 @@ def test_qk_norm_rope_and_cache_append(capi, torch, n_q, n_kv, pos):
     assert (kc[pos].cpu().float() - kh[0, :, 0].float()).abs().max() <= 0.03 * max(k_ref.abs().max().item(), 1.0)
 
 
+@pytest.mark.parametrize("pos", [4, 5, 1 << 20, -1, -(1 << 31)])
+def test_cache_append_skips_positions_outside_the_cache(capi, torch, pos):
+    """A position the caches have no row for writes nothing into them (memory on either side of the
+    caches keeps its contents); the query heads are still produced."""
+    n_q, n_kv, D, rows = 4, 2, 128, 4
+    qkv = torch.randn((n_q + 2 * n_kv) * D).bfloat16().cuda()
+    g = torch.ones(D, dtype=torch.bfloat16, device="cuda")
+    q_out = torch.full((n_q, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    # the caches sit in the middle of a larger buffer: rows before and after them must stay as they are
+    pool = torch.full((2, rows + 4, n_kv, D), 7.0, dtype=torch.bfloat16, device="cuda")
+    kc, vc = pool[0, 2:2 + rows], pool[1, 2:2 + rows]
+    capi.qk_norm_rope_bf16(qkv, g, g, q_out, kc, vc, n_q, n_kv,
+                           torch.tensor([pos], dtype=torch.int32, device="cuda"), 1e6, 1e-6)
+    torch.cuda.synchronize()
+    assert (pool == 7.0).all()
+    assert torch.isfinite(q_out.float()).all()
+
+
 @pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (8, 4), (4, 4)])
 @pytest.mark.parametrize("ctx", [1, 5, 128, 129, 1000, 4097])
 def test_attention_decode_matches_fp32_softmax(capi, torch, n_q, n_kv, ctx):

@@ -206,6 +206,14 @@ def test_qkv_rope_launch_equals_separate_launches(capi, torch, K, n_q, n_kv, gro
     assert (k_one[:pos_value] == 3.0).all() and (k_one[pos_value + 1:] == 3.0).all()
     assert (v_one[:pos_value] == 5.0).all() and (v_one[pos_value + 1:] == 5.0).all()
     assert torch.isfinite(q_one.float()).all()
+    # a position the caches have no row for: nothing is appended
+    k_off, v_off = caches()
+    for bad in (max_pos, -1):
+        capi.gemv_awq_qkv_rope_bf16(resid, delta, gain, eps, r_one, qw, sc, qz, q_gain, k_gain, q_one, k_off, v_off,
+                                    n_q, n_kv, torch.tensor([bad], dtype=torch.int32, device="cuda"), theta, eps,
+                                    group, ws)
+    torch.cuda.synchronize()
+    assert (k_off == 3.0).all() and (v_off == 5.0).all()
 
 
 def test_qkv_rope_launch_rejects_bad_arguments(capi, torch):
