@@ -253,9 +253,10 @@ int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const in
  *                         0 .. cache_positions-1 writes no cache row).  head_dim must be 128.
  *   kx_attn_decode_bf16   GQA attention of one query position against cache rows 0 .. *pos:
  *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv in
- *                         {1,2,4,8}; split over the context in chunks of 64 positions, merged by
- *                         log-sum-exp.  `max_positions` (<= 32768) fixes the launch shape (a captured
- *                         graph can be replayed while *pos advances up to max_positions - 1).
+ *                         {1,2,4,8}; split over the context in chunks, merged by log-sum-exp.
+ *                         `max_positions` (<= 65536) fixes the launch shape (a captured graph can be
+ *                         replayed while *pos advances up to max_positions - 1) and the chunk size:
+ *                         64 positions up to max_positions = 5120, 128 beyond.
  *   kx_attn_decode_partial_bf16   the first stage only: the per-chunk results stay in the workspace for
  *                         kx_gemv_awq_attn_merge_bf16 (below) to merge inside the o projection.
  *   kx_swiglu_bf16        out = bf16(silu(gate)) * up
@@ -283,7 +284,7 @@ int kx_attn_decode_partial_bf16(const uint16_t* q, const uint16_t* k_cache, cons
  * y = attn W, where attn [n_q_heads * 128] is what kx_attn_decode_bf16 would have written, merged
  * here from the workspace that kx_attn_decode_partial_bf16 filled with the same n_q_heads, n_kv_heads
  * and max_positions.  Bitwise the result of kx_attn_decode_bf16 followed by kx_gemv_awq_bf16 on the
- * vector kernel.  max_positions <= 5120 (80 chunks: a thread holds a row's per-chunk values in
+ * vector kernel.  max_positions <= 10240 (80 chunks: a thread holds a row's per-chunk values in
  * registers); longer contexts use the two separate calls.
  * Replaces: the tail of LayerMHA + LayerMatmul back to back (kuiper/include/op/layer.h:8-20). */
 int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t attn_workspace_bytes, int32_t n_q_heads,

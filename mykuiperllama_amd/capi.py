@@ -258,7 +258,7 @@ def gemv_awq_chain_bf16(desc, qweight, scales, qzeros, K, N, group_size, workspa
                                          _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream()))
 
 
-FUSED_MERGE_MAX_POSITIONS = 80 * 64  # the o projection merges at most 80 chunks of 64 positions
+FUSED_MERGE_MAX_POSITIONS = 80 * 128  # the o projection merges at most 80 chunks (of 128 positions past 5120)
 
 
 def swiglu_bf16(gate, up, out):

@@ -14,7 +14,18 @@
 
 namespace kx {
 
-constexpr int kAttnChunk = 64;      // cache positions per chunk of the first stage
+// Cache positions per chunk of the first stage: 64 for caches of up to 5120 positions (more, smaller
+// workgroups: the first stage is a chain of latencies), 128 beyond, which keeps the number of chunks
+// of a cache of up to 10240 positions within what the o projection can merge in its prologue.
+constexpr int kAttnChunkShort = 64;
+constexpr int kAttnChunkLong = 128;
+constexpr int kAttnShortLimit = 80 * kAttnChunkShort;
+__host__ __device__ constexpr int attn_chunk_for(int max_positions) {
+    return max_positions <= kAttnShortLimit ? kAttnChunkShort : kAttnChunkLong;
+}
+__host__ __device__ constexpr int attn_chunks_of(int max_positions) {
+    return (max_positions + attn_chunk_for(max_positions) - 1) / attn_chunk_for(max_positions);
+}
 constexpr int kMergeParts = 4;      // a dimension is summed over the chunks c = p, p + 4, ... for p = 0..3 side by side
 constexpr int kMergeBatch = 8;      // loads in flight per thread in the stand-alone merge
 constexpr int kMergeLanesLong = 8;  // chunks per lane the stand-alone merge provides for: 512 chunks

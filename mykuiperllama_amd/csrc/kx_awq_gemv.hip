@@ -380,7 +380,7 @@ extern "C" int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t at
     const int K = n_q_heads * kx::kHeadDim;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, 1, K, N, group_size);
     if (rc != KX_OK) return rc;
-    const int nchunks = (max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    const int nchunks = kx::attn_chunks_of(max_positions);
     // a thread holds kMergeHold values of each of its elements: longer contexts take the separate merge
     if (nchunks > kx::kMergeParts * kx::kMergeHold) return KX_ERR_BAD_SHAPE;
     const size_t need = static_cast<size_t>(nchunks) * n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
@@ -460,7 +460,7 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
                 K != d->n_q_heads * kx::kHeadDim) {
                 return KX_ERR_BAD_SHAPE;
             }
-            const int nchunks = (d->max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
+            const int nchunks = kx::attn_chunks_of(d->max_positions);
             if (nchunks > kx::kMergeParts * kx::kMergeHold) return KX_ERR_BAD_SHAPE;
             const size_t need = static_cast<size_t>(nchunks) * d->n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
             if (d->attn_workspace_bytes < need) return KX_ERR_WORKSPACE;

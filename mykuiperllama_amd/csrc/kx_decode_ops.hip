@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 
 // ------------------------------------------------------------------------------------------------
 // GQA flash-decoding, head_dim 128, one query position.
-// Stage 1: a workgroup takes one KV head and one chunk of kAttnChunk cache positions and serves the
+// Stage 1: a workgroup takes one KV head and one chunk of CHUNK (64 or 128) cache positions and serves the
 // G = n_q / n_kv query heads of that KV head together, so every K and V row is read once.  Sixteen
 // lanes share a position (eight dims each, one contiguous 256-byte row per position); a wave walks
 // four positions per load.  Scores go to LDS, softmax statistics are taken per head over the chunk,
@@ -132,17 +132,17 @@ constexpr int kAttnSlots = kAttnThreads / 16;  // cache positions a workgroup ha
 constexpr int kAccHeads = 4;                   // heads whose slot sums fit in LDS together (32 KiB)
 constexpr int kMaxGroup = 8;  // query heads per KV head this kernel is instantiated for
 
-template <int G>
+template <int G, int CHUNK>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, const int32_t* __restrict__ pos_ptr,
     int nchunks, int max_positions, float scale) {
-    __shared__ float s_score[G][kAttnChunk];
+    __shared__ float s_score[G][CHUNK];
     __shared__ __attribute__((aligned(16))) float s_acc[kAttnSlots][G < kAccHeads ? G : kAccHeads][kHeadDim];
 
     const int kvh = blockIdx.y;
     const int chunk = blockIdx.x;
-    const int p0 = chunk * kAttnChunk;
+    const int p0 = chunk * CHUNK;
     const int tid = threadIdx.x;
     const int sub = tid % 16;    // which eight dims of the row
     const int slot = tid / 16;   // position slot inside the workgroup: 16 slots
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // not depend on *pos: any row below max_positions exists, rows past the context are masked once
     // the position has arrived.  The chunk then costs one memory round trip.
     const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
-    constexpr int ITERS = kAttnChunk / 16;
+    constexpr int ITERS = CHUNK / 16;
     // The G query heads, this lane's eight dims of each, are requested first: loads return in order,
     // and the scores need q and K but not V, so q must not queue behind the V rows.
     uint4 qraw[G];
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // softmax statistics per head over the chunk; wave w serves heads w, w + 4, ...
     for (int g = tid / kWave; g < G; g += kAttnThreads / kWave) {
         const int lane = tid % kWave;
-        constexpr int PER_LANE = kAttnChunk / kWave;
+        constexpr int PER_LANE = CHUNK / kWave;
         float sc[PER_LANE];
         float m = -INFINITY;
 #pragma unroll
@@ -482,7 +482,7 @@ extern "C" int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain,
 
 extern "C" size_t kx_attn_decode_workspace_bytes(int32_t n_q_heads, int32_t head_dim, int32_t max_positions) {
     if (n_q_heads < 1 || head_dim != kx::kHeadDim || max_positions < 1) return 0;
-    const size_t nchunks = (static_cast<size_t>(max_positions) + kx::kAttnChunk - 1) / kx::kAttnChunk;
+    const size_t nchunks = static_cast<size_t>(kx::attn_chunks_of(max_positions));
     return nchunks * n_q_heads * (kx::kHeadDim + 2) * sizeof(float);
 }
 
@@ -502,16 +502,24 @@ int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_ca
     if (!kx::aligned16(q) || !kx::aligned16(k_cache) || !kx::aligned16(v_cache) || !kx::aligned16(workspace)) {
         return KX_ERR_ALIGNMENT;
     }
-    const int nchunks = (max_positions + kx::kAttnChunk - 1) / kx::kAttnChunk;
-    if (nchunks > kx::kMergeLanesLong * kx::kWave) return KX_ERR_BAD_SHAPE;  // 32768 positions
+    const int nchunks = kx::attn_chunks_of(max_positions);
+    if (nchunks > kx::kMergeLanesLong * kx::kWave) return KX_ERR_BAD_SHAPE;  // 65536 positions
+    const bool long_chunks = kx::attn_chunk_for(max_positions) == kx::kAttnChunkLong;
     float* part_out = static_cast<float*>(workspace);
     float* part_ml = part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
     const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
     hipStream_t s = kx::as_stream(stream);
     dim3 grid1(nchunks, n_kv_heads);
 #define KX_ATTN(GG)                                                                                             \
-    hipLaunchKernelGGL((kx::attn_decode_stage1<GG>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache, v_cache,  \
-                       part_out, part_ml, n_kv_heads, pos, nchunks, max_positions, scale);                      \
+    if (long_chunks) {                                                                                          \
+        hipLaunchKernelGGL((kx::attn_decode_stage1<GG, kx::kAttnChunkLong>), grid1, dim3(kx::kAttnThreads), 0,  \
+                           s, q, k_cache, v_cache, part_out, part_ml, n_kv_heads, pos, nchunks, max_positions,  \
+                           scale);                                                                              \
+    } else {                                                                                                    \
+        hipLaunchKernelGGL((kx::attn_decode_stage1<GG, kx::kAttnChunkShort>), grid1, dim3(kx::kAttnThreads), 0, \
+                           s, q, k_cache, v_cache, part_out, part_ml, n_kv_heads, pos, nchunks, max_positions,  \
+                           scale);                                                                              \
+    }                                                                                                           \
     if (out) {                                                                                                  \
         hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kMergeThreads),              \
                            nchunks * sizeof(float), s, part_out, part_ml, out, nchunks);                        \

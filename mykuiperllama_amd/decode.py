@@ -60,11 +60,19 @@ def _rand_awq(torch, K, N, group, gen):
 class DecodeModel:
     """Weights, caches and scratch buffers of one model on the GPU."""
 
-    def __init__(self, cfg, max_positions, weights=None, seed=20251125):
+    def __init__(self, cfg, max_positions, weights=None, seed=20251125, merge_in_o=None):
         import torch
         self.torch = torch
         self.cfg = cfg
         self.max_positions = max_positions
+        # Where the attention chunks are merged: in the prologue of the o projection (one launch
+        # fewer per layer) when the cache is short enough for it.  Every workgroup of that projection
+        # repeats the merge of its two heads, so it pays while the projection has about one round of
+        # workgroups (Qwen3-8B: 256 of them, 1.5 us per layer faster; Qwen3-32B: 640, 2 us slower
+        # than the separate merge kernel).  The caller can decide otherwise.
+        fits = max_positions <= capi.FUSED_MERGE_MAX_POSITIONS
+        o_workgroups = -(-cfg.hidden // 256) * max(1, cfg.n_q * cfg.head_dim // 256)
+        self.merge_in_o = fits and (o_workgroups <= 512 if merge_in_o is None else bool(merge_in_o))
         c = cfg
         gen = torch.Generator(device="cuda")
         gen.manual_seed(seed)
@@ -184,7 +192,7 @@ class DecodeModel:
             capi.gemv_awq_qkv_rope_bf16(xa, None if li == 0 else self.down, L["in_norm"], c.eps, xb, qw, sc, qz,
                                         L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
                                         c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps, g, ws)
-            if self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS:
+            if self.merge_in_o:
                 capi.attn_decode_partial_bf16(self.q, self.k_cache[li], self.v_cache[li], c.n_q, c.n_kv, self.pos,
                                               self.max_positions, self.attn_ws)
                 qw, sc, qz = L["o"]
@@ -208,7 +216,7 @@ class DecodeModel:
         c = self.cfg
         g, ws = c.group, self.gemv_ws
         H, I = c.hidden, c.intermediate
-        merge_in_o = self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS
+        merge_in_o = self.merge_in_o
         capi.embedding_bf16(self.embed, self.token, self.x)
         x, ssq = self.x, self.ssq
         rope = {"out_kind": capi.OUT_QKV_ROPE, "q_out": self.q, "pos": self.pos, "rope_n_q_heads": c.n_q,
@@ -253,7 +261,7 @@ class DecodeModel:
     def launches_per_step(self, with_lm_head=True, fused=True):
         per_layer = 10
         if fused:
-            per_layer = 5 if self.max_positions <= capi.FUSED_MERGE_MAX_POSITIONS else 6
+            per_layer = 5 if self.merge_in_o else 6
         return 1 + self.cfg.layers * per_layer + 1 + (2 if with_lm_head else 0)
 
 

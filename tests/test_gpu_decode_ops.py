@@ -139,10 +139,12 @@ def test_cache_append_skips_positions_outside_the_cache(capi, torch, pos):
 
 
 @pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (8, 4), (4, 4)])
-@pytest.mark.parametrize("ctx", [1, 5, 128, 129, 1000, 4097])
-def test_attention_decode_matches_fp32_softmax(capi, torch, n_q, n_kv, ctx):
+@pytest.mark.parametrize("ctx,max_pos", [(1, 4224), (5, 4224), (128, 4224), (129, 4224), (1000, 4224), (4097, 4224),
+                                         # caches past 5120 positions are walked in chunks of 128
+                                         (1, 5121), (127, 8320), (128, 8320), (129, 8320), (8193, 8320),
+                                         (12000, 12032)])
+def test_attention_decode_matches_fp32_softmax(capi, torch, n_q, n_kv, ctx, max_pos):
     D = 128
-    max_pos = 4224
     G = n_q // n_kv
     q = torch.randn(n_q, D).bfloat16()
     kc = torch.randn(max_pos, n_kv, D).bfloat16()

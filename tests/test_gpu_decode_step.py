@@ -195,6 +195,27 @@ def test_chained_step_agrees_with_the_prologue_step_to_rounding(torch):
     assert (ka - kb).abs().max().item() <= 0.05
 
 
+@pytest.mark.parametrize("max_pos,ctx", [(48, 37), (6000, 5500), (10240, 10239), (10368, 7000)])
+def test_merge_inside_the_o_projection_or_as_a_launch_of_its_own_is_the_same_step(torch, max_pos, ctx):
+    """Where the attention chunks are merged changes nothing, bit for bit; caches past 5120 positions are
+    walked in chunks of 128, past 10240 the merge is always a launch of its own."""
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    results = []
+    for merge_in_o in (True, False):
+        model = decode.DecodeModel(cfg, max_pos, merge_in_o=merge_in_o)
+        assert model.merge_in_o == (merge_in_o and max_pos <= 10240)
+        model.prefill_cache_random(ctx)
+        model.set_input(9, ctx)
+        model.step(fused="chain")
+        torch.cuda.synchronize()
+        assert torch.isfinite(model.logits.float()).all()
+        results.append((model.logits.clone(), model.x.clone()))
+        assert model.launches_per_step(True) == 4 + cfg.layers * (5 if model.merge_in_o else 6)
+    for a, b in zip(*results):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
 @pytest.mark.parametrize("fused", [True, "prologue", False])
 def test_step_is_capturable_in_a_graph_and_replays_identically(torch, fused):
     """A captured step replayed with the same inputs gives bitwise the same logits as eager."""

@@ -245,7 +245,10 @@ MERGE_CASES = [
     # n_q, n_kv, pos, max_positions, N, group
     (32, 8, 4096, 4224, 4096, 128),   # Qwen3-8B at the benchmark's context
     (32, 8, 0, 4224, 4096, 128),      # a single cached position
-    (32, 8, 63, 5120, 1024, 128),     # the longest context the merging projection takes
+    (32, 8, 63, 5120, 1024, 128),     # the longest cache walked in chunks of 64 positions
+    (64, 8, 8192, 8320, 5120, 128),   # Qwen3-32B at its benchmark context: chunks of 128 positions
+    (8, 2, 10239, 10240, 512, 128),   # the longest context the merging projection takes
+    (8, 2, 5000, 5121, 512, 128),     # just past the switch to chunks of 128
     (64, 8, 1000, 1100, 5120, 128),   # eight query heads per KV head
     (4, 2, 37, 48, 512, 128),
     (2, 1, 100, 128, 264, 32),        # K = 256, ragged N
@@ -291,9 +294,9 @@ def test_attention_merge_rejects_long_contexts_and_bad_arguments(capi, torch):
     _, (qw, sc, qz) = weights(torch, "fused_merge_bad", 1, n_q * 128, N, group)
     y = torch.zeros((1, N), dtype=torch.bfloat16, device="cuda")
     ws = capi.make_workspace(1, n_q * 128, N)
-    long_ws = capi.attn_decode_workspace(n_q, 5121)
+    long_ws = capi.attn_decode_workspace(n_q, 10241)
     with pytest.raises(capi.KxError) as e:
-        capi.gemv_awq_attn_merge_bf16(long_ws, n_q, n_kv, 5121, qw, sc, qz, y, group, ws)
+        capi.gemv_awq_attn_merge_bf16(long_ws, n_q, n_kv, 10241, qw, sc, qz, y, group, ws)
     assert e.value.code == -2
     small_ws = capi.attn_decode_workspace(n_q, 64)
     with pytest.raises(capi.KxError) as e:
