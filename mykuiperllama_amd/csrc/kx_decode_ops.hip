@@ -374,65 +374,72 @@ __global__ __launch_bounds__(256) void embedding_kernel(const uint16_t* __restri
 }
 
 // argmax over n bf16 values, first index on ties, NaN ignored; one workgroup.
+// Two passes, because one compute unit's vector ALUs are what bounds it: the first takes the maximum
+// alone (one v_max per element instead of two compares and two selects), the second looks for the
+// first index that holds it, and only in the threads whose own maximum is the overall one.
 constexpr int kArgmaxThreads = 1024;
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* __restrict__ x, int n,
                                                                int32_t* __restrict__ out) {
-    __shared__ float s_val[kArgmaxThreads / kWave];
-    __shared__ int s_idx[kArgmaxThreads / kWave];
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    auto consider = [&](float v, int i) {
-        // strictly greater, or equal with a smaller index: the first maximum wins; NaN never wins
-        if (v > best || (v == best && i < best_i)) {
-            best = v;
-            best_i = i;
-        }
-    };
+    constexpr int kWaves = kArgmaxThreads / kWave;
+    __shared__ float s_val[kWaves];
+    __shared__ int s_idx[kWaves];
+    const int tid = threadIdx.x;
     const bool wide = (reinterpret_cast<uintptr_t>(x) % 16) == 0;
     const int chunks = wide ? n / 8 : 0;
+    const uint4* xv = reinterpret_cast<const uint4*>(x);
+
+    float mine = -INFINITY;  // fmaxf drops a NaN operand
     constexpr int kInFlight = 8;  // 16-byte loads per thread and sweep
-    for (int c0 = threadIdx.x; c0 < chunks; c0 += kInFlight * kArgmaxThreads) {
+    for (int c0 = tid; c0 < chunks; c0 += kInFlight * kArgmaxThreads) {
         // clamped addresses: the loads of a sweep are straight-line code, all in flight together;
-        // a piece past the end is looked at with values and indices that can never win
+        // a piece past the end re-reads the last one, which cannot change a maximum
         uint4 raw[kInFlight];
 #pragma unroll
         for (int u = 0; u < kInFlight; u++) {
             const int c = c0 + u * kArgmaxThreads;
-            raw[u] = reinterpret_cast<const uint4*>(x)[c < chunks ? c : chunks - 1];
+            raw[u] = xv[c < chunks ? c : chunks - 1];
         }
 #pragma unroll
         for (int u = 0; u < kInFlight; u++) {
-            const int c = c0 + u * kArgmaxThreads;
-            const bool live = c < chunks;
             float v[8];
             unpack8(raw[u], v);
 #pragma unroll
-            for (int i = 0; i < 8; i++) consider(live ? v[i] : -INFINITY, live ? 8 * c + i : 0x7fffffff);
+            for (int i = 0; i < 8; i++) mine = fmaxf(mine, v[i]);
         }
     }
-    for (int i = 8 * chunks + threadIdx.x; i < n; i += kArgmaxThreads) consider(bf16_to_f32(x[i]), i);
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(best, off, kWave);
-        const int oi = __shfl_xor(best_i, off, kWave);
-        if (ov > best || (ov == best && oi < best_i)) {
-            best = ov;
-            best_i = oi;
-        }
-    }
-    if (threadIdx.x % kWave == 0) {
-        s_val[threadIdx.x / kWave] = best;
-        s_idx[threadIdx.x / kWave] = best_i;
-    }
+    for (int i = 8 * chunks + tid; i < n; i += kArgmaxThreads) mine = fmaxf(mine, bf16_to_f32(x[i]));
+    const float wave_best = wave_max(mine);
+    if (tid % kWave == 0) s_val[tid / kWave] = wave_best;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < kArgmaxThreads / kWave; w++) {
-            if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
-                best = s_val[w];
-                best_i = s_idx[w];
+    float best = s_val[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) best = fmaxf(best, s_val[w]);
+
+    int first = 0x7fffffff;
+    if (mine == best) {  // few threads: they walk their own elements again (-0 and +0 are one value)
+        for (int c = tid; c < chunks; c += kArgmaxThreads) {
+            float v[8];
+            unpack8(xv[c], v);
+#pragma unroll
+            for (int i = 7; i >= 0; i--) {
+                if (v[i] == best && 8 * c + i < first) first = 8 * c + i;
             }
         }
-        out[0] = best_i == 0x7fffffff ? 0 : best_i;
+        for (int i = 8 * chunks + tid; i < n; i += kArgmaxThreads) {
+            if (bf16_to_f32(x[i]) == best && i < first) first = i;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const int other = __shfl_xor(first, off, kWave);
+        first = other < first ? other : first;
+    }
+    if (tid % kWave == 0) s_idx[tid / kWave] = first;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) first = s_idx[w] < first ? s_idx[w] : first;
+        out[0] = first == 0x7fffffff ? 0 : first;  // nothing but NaN: index 0
     }
 }
 

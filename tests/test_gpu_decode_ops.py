@@ -203,6 +203,16 @@ def test_swiglu_add_embedding_argmax(capi, torch):
     capi.argmax_bf16(logits.cuda(), idx)
     torch.cuda.synchronize()
     assert idx.item() == 123
+    for fill, want in ((float("nan"), 0), (float("-inf"), 0), (-0.0, 0)):
+        flat = torch.full((4099,), fill).bfloat16()
+        capi.argmax_bf16(flat.cuda(), idx)
+        torch.cuda.synchronize()
+        assert idx.item() == want
+    flat = torch.full((4099,), -1.0).bfloat16()
+    flat[4000], flat[4098] = -0.0, 0.0  # the two zeros are one value: the first of them wins
+    capi.argmax_bf16(flat.cuda(), idx)
+    torch.cuda.synchronize()
+    assert idx.item() == 4000
     # ragged lengths (shorter than one 16-byte piece, not a multiple of eight, the maximum in the
     # last element) and a pointer off the 16-byte grid
     g = torch.Generator().manual_seed(5)
