@@ -44,31 +44,44 @@ __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
 #pragma unroll
     for (int m = 0; m < MB; m++) acc[m] = 0.0f;
 
-    for (int c0 = lane; c0 < chunks; c0 += kWave * kUnroll) {
-        // Clamped addresses, masked weights: the loads of a sweep are straight-line code and all
-        // in flight together (a load under a condition becomes a branch with a full wait behind it).
+    // Full sweeps of kUnroll pieces per lane, then the rest of the row two pieces per lane at a time
+    // (K = 5120: one full sweep and one short one).  Inside a sweep the loads are straight-line code
+    // and all in flight together; a load under a condition becomes a branch with a full wait behind it.
+    auto consume = [&](const u32x4& wv, int c, bool live) {
+        const uint32_t w0 = live ? wv.x : 0u, w1 = live ? wv.y : 0u;
+        const uint32_t w2 = live ? wv.z : 0u, w3 = live ? wv.w : 0u;
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            const uint4 xv = xrow[m][c];
+            acc[m] = dot2_bf16(w0, xv.x, acc[m]);
+            acc[m] = dot2_bf16(w1, xv.y, acc[m]);
+            acc[m] = dot2_bf16(w2, xv.z, acc[m]);
+            acc[m] = dot2_bf16(w3, xv.w, acc[m]);
+        }
+    };
+    int base = 0;  // first piece of the sweep, the same in every lane
+    for (; base + kWave * kUnroll <= chunks; base += kWave * kUnroll) {
         u32x4 wv[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-            const int c = c0 + u * kWave;
-            wv[u] = __builtin_nontemporal_load(wrow + (c < chunks ? c : chunks - 1));
-        }
+        for (int u = 0; u < kUnroll; u++) wv[u] = __builtin_nontemporal_load(wrow + base + lane + u * kWave);
         __builtin_amdgcn_sched_barrier(0);  // every weight load is out before the first is waited for
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-            const int c = c0 + u * kWave;
-            const bool live = c < chunks;
-            const int cl = live ? c : chunks - 1;
-            const uint32_t w0 = live ? wv[u].x : 0u, w1 = live ? wv[u].y : 0u;
-            const uint32_t w2 = live ? wv[u].z : 0u, w3 = live ? wv[u].w : 0u;
+        for (int u = 0; u < kUnroll; u++) consume(wv[u], base + lane + u * kWave, true);
+    }
+    constexpr int kTail = 2;
+    for (; base < chunks; base += kWave * kTail) {
+        // clamped addresses, masked weights
+        u32x4 wv[kTail];
 #pragma unroll
-            for (int m = 0; m < MB; m++) {
-                const uint4 xv = xrow[m][cl];
-                acc[m] = dot2_bf16(w0, xv.x, acc[m]);
-                acc[m] = dot2_bf16(w1, xv.y, acc[m]);
-                acc[m] = dot2_bf16(w2, xv.z, acc[m]);
-                acc[m] = dot2_bf16(w3, xv.w, acc[m]);
-            }
+        for (int u = 0; u < kTail; u++) {
+            const int c = base + lane + u * kWave;
+            wv[u] = __builtin_nontemporal_load(wrow + (c < chunks ? c : chunks - 1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < kTail; u++) {
+            const int c = base + lane + u * kWave;
+            consume(wv[u], c < chunks ? c : chunks - 1, c < chunks);
         }
     }
 #pragma unroll
