@@ -30,21 +30,11 @@
 
 namespace kx {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4v __attribute__((ext_vector_type(4)));
-
 constexpr int kStepRows = 32;  // rows of K per MFMA step
 
 // Column (0..7) inside a word -> nibble that holds it (inverse of order_of).
 __host__ __device__ constexpr int nibble_of(int col) {
     return (col & 1) ? 4 + (col >> 1) : (col >> 1);
-}
-
-__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-    u32x4 v = {a, b, c, d};
-    bf16x8 out;
-    __builtin_memcpy(&out, &v, 16);
-    return out;
 }
 
 // Two bf16 128.0 in a register whose value the compiler cannot see.  (v & 0x000F000F) | magic then

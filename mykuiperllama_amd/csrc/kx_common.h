@@ -56,6 +56,18 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return static_cast<float>(v);
 }
 
+// Operand and result types of v_mfma_f32_16x16x32_bf16: lane l supplies eight consecutive k
+// (8*(l/16) .. +7) of row (A) or column (B) l%16 and receives D[4*(l/16)+v][l%16], v = 0..3.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    u32x4 v = {a, b, c, d};
+    bf16x8 out;
+    __builtin_memcpy(&out, &v, 16);
+    return out;
+}
+
 // Lane exchanges inside a row of 16 lanes ride on the VALU's data-parallel-primitive operand path
 // (one instruction for move + add), where a ds_bpermute costs an LDS round trip of ~100 cycles that a
 // dependent chain cannot hide.  CTRL 0x120 + n rotates a row right by n lanes.

@@ -120,10 +120,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 // ------------------------------------------------------------------------------------------------
 // GQA flash-decoding, head_dim 128, one query position.
 // Stage 1: a workgroup takes one KV head and one chunk of CHUNK (64 or 128) cache positions and serves the
-// G = n_q / n_kv query heads of that KV head together, so every K and V row is read once.  Sixteen
-// lanes share a position (eight dims each, one contiguous 256-byte row per position); a wave walks
-// four positions per load.  Scores go to LDS, softmax statistics are taken per head over the chunk,
-// then V is accumulated with the chunk-local weights.  Output per (KV head, chunk): for each of the
+// G = n_q / n_kv query heads of that KV head together, so every K and V row is read once.  The
+// scores q . K come from the matrix cores, sixteen positions per tile; they go to LDS, softmax
+// statistics are taken per head over the chunk, then V is accumulated with the chunk-local weights
+// on the vector ALUs: sixteen lanes share a position (eight dims each, one contiguous 256-byte row
+// per position), a wave walks four positions per load.  Output per (KV head, chunk): for each of the
 // G heads the unnormalised 128-vector, the chunk maximum and the chunk sum of exponentials.
 // Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
 // ------------------------------------------------------------------------------------------------
@@ -152,20 +153,34 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // the position has arrived.  The chunk then costs one memory round trip.
     const size_t row_stride = static_cast<size_t>(n_kv) * kHeadDim;  // elements between positions
     constexpr int ITERS = CHUNK / 16;
-    // The G query heads, this lane's eight dims of each, are requested first: loads return in order,
-    // and the scores need q and K but not V, so q must not queue behind the V rows.
-    uint4 qraw[G];
+    // Scores on the matrix cores: per tile of sixteen positions, D[head][position] = sum over the 128
+    // dims in four steps of 32, A = the query heads (row = head, zero rows past G), B = the K rows
+    // (column = position).  Lane (c = lane % 16, b = lane / 16) supplies dims 32 s + 8 b .. + 7 of head
+    // c and of position c, sixteen contiguous bytes each.  A wave takes TPW of the chunk's tiles.
+    constexpr int kWaves = kAttnThreads / kWave;
+    constexpr int TPW = ITERS / kWaves;  // position tiles per wave: 1 (chunks of 64) or 2 (128)
+    static_assert(ITERS % kWaves == 0, "whole tiles per wave");
+    const int wave = tid / kWave;
+    const int mc = (tid % kWave) % 16;
+    const int mb = (tid % kWave) / 16;
+    // The query heads are requested first: loads return in order, and the scores need q and K but
+    // not V, so q must not queue behind the V rows.
+    u32x4 qraw[4];
+    const int q_head = mc < G ? mc : G - 1;  // clamped: rows past G are zeroed below
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-        qraw[g] = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(kvh) * G + g) * kHeadDim + 8 * sub);
+    for (int ks = 0; ks < 4; ks++) {
+        qraw[ks] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(kvh) * G + q_head) * kHeadDim + 32 * ks + 8 * mb);
     }
-    u32x4 kraw[ITERS], vraw[ITERS];
+    u32x4 kraw[TPW][4], vraw[ITERS];
 #pragma unroll
-    for (int it = 0; it < ITERS; it++) {
-        const int p = p0 + it * 16 + slot;
+    for (int t = 0; t < TPW; t++) {
+        const int p = p0 + (wave * TPW + t) * 16 + mc;
         const int pc = p < max_positions ? p : max_positions - 1;
-        kraw[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
-            k_cache + pc * row_stride + static_cast<size_t>(kvh) * kHeadDim + 8 * sub));
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            kraw[t][ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                k_cache + pc * row_stride + static_cast<size_t>(kvh) * kHeadDim + 32 * ks + 8 * mb));
+        }
     }
 #pragma unroll
     for (int it = 0; it < ITERS; it++) {
@@ -176,9 +191,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     }
     const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
     __builtin_amdgcn_sched_barrier(0);
-    float qv[G][8];
-#pragma unroll
-    for (int g = 0; g < G; g++) unpack8(qraw[g], qv[g]);
 
     float* out_base = part_out + (static_cast<size_t>(kvh) * nchunks + chunk) * G * kHeadDim;
     float* ml_base = part_ml + (static_cast<size_t>(kvh) * nchunks + chunk) * G * 2;
@@ -188,18 +200,23 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // everything masked and reports max = -inf, sum = 0.
 
     // pass 1: scores
+    const bool q_live = mc < G;
 #pragma unroll
-    for (int it = 0; it < ITERS; it++) {
-        const int p = p0 + it * 16 + slot;
-        float kd[8];
-        unpack8(make_uint4(kraw[it].x, kraw[it].y, kraw[it].z, kraw[it].w), kd);
+    for (int t = 0; t < TPW; t++) {
+        f32x4v d = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            float d = 0.0f;
+        for (int ks = 0; ks < 4; ks++) {
+            const bf16x8 a_op = as_bf16x8(q_live ? qraw[ks].x : 0u, q_live ? qraw[ks].y : 0u,
+                                          q_live ? qraw[ks].z : 0u, q_live ? qraw[ks].w : 0u);
+            const bf16x8 b_op = as_bf16x8(kraw[t][ks].x, kraw[t][ks].y, kraw[t][ks].z, kraw[t][ks].w);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, b_op, d, 0, 0, 0);
+        }
+        // the lane holds heads 4 mb .. 4 mb + 3 of position mc of the tile
+        const int pl = (wave * TPW + t) * 16 + mc;
 #pragma unroll
-            for (int i = 0; i < 8; i++) d = __builtin_fmaf(qv[g][i], kd[i], d);
-            d = row16_sum(d);  // the sixteen lanes of the position
-            if (sub == 0) s_score[g][it * 16 + slot] = (p < ctx) ? d * scale : -INFINITY;
+        for (int v = 0; v < 4; v++) {
+            const int head = 4 * mb + v;
+            if (head < G) s_score[head][pl] = (p0 + pl < ctx) ? d[v] * scale : -INFINITY;
         }
     }
     __syncthreads();
