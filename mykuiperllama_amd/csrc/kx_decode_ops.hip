@@ -122,15 +122,13 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 // Stage 1: a workgroup takes one KV head and one chunk of CHUNK (64 or 128) cache positions and serves the
 // G = n_q / n_kv query heads of that KV head together, so every K and V row is read once.  The
 // scores q . K come from the matrix cores, sixteen positions per tile; they go to LDS, softmax
-// statistics are taken per head over the chunk, then V is accumulated with the chunk-local weights
-// on the vector ALUs: sixteen lanes share a position (eight dims each, one contiguous 256-byte row
-// per position), a wave walks four positions per load.  Output per (KV head, chunk): for each of the
+// statistics are taken per head over the chunk, then the V rows (loaded sixteen lanes per position,
+// one contiguous 256-byte row each, and staged in LDS) are accumulated with the chunk-local weights,
+// again on the matrix cores.  Output per (KV head, chunk): for each of the
 // G heads the unnormalised 128-vector, the chunk maximum and the chunk sum of exponentials.
 // Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnThreads = 256;
-constexpr int kAttnSlots = kAttnThreads / 16;  // cache positions a workgroup handles side by side
-constexpr int kAccHeads = 4;                   // heads whose slot sums fit in LDS together (32 KiB)
 constexpr int kMaxGroup = 8;  // query heads per KV head this kernel is instantiated for
 
 template <int G, int CHUNK>
@@ -138,8 +136,14 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, const int32_t* __restrict__ pos_ptr,
     int nchunks, int max_positions, float scale) {
-    __shared__ float s_score[G][CHUNK];
-    __shared__ __attribute__((aligned(16))) float s_acc[kAttnSlots][G < kAccHeads ? G : kAccHeads][kHeadDim];
+    // Scores, then softmax weights, per head; rows padded so that the sixteen-byte reads of the
+    // second pass (one row per lane) do not all start on the same bank.
+    __shared__ __attribute__((aligned(16))) float s_score[G][CHUNK + 4];
+    // The chunk's V rows, row-major, one dword of padding per row: the second pass reads them
+    // transposed (eight positions of one dim per lane), and with 65 dwords per row the four blocks of
+    // eight positions that a read instruction touches fall on different banks.
+    constexpr int kVRow = kHeadDim / 2 + 1;
+    __shared__ uint32_t s_v[CHUNK][kVRow];
 
     const int kvh = blockIdx.y;
     const int chunk = blockIdx.x;
@@ -247,52 +251,70 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
             ml_base[2 * g + 1] = l;
         }
     }
-    __syncthreads();
-
-    // pass 2: weighted sum of V rows
-    float acc[G][8];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
-    }
+    // The V rows go to LDS while the statistics are being taken: rows past the context carry weight 0,
+    // their (arbitrary) contents are zeroed so that a stray NaN or infinity cannot leak through 0 * x.
 #pragma unroll
     for (int it = 0; it < ITERS; it++) {
-        // rows past the context carry weight 0; their (arbitrary) contents are zeroed so that a stray
-        // NaN or infinity cannot leak through 0 * x
-        const bool live = p0 + it * 16 + slot < ctx;
-        float vd[8];
-        unpack8(live ? make_uint4(vraw[it].x, vraw[it].y, vraw[it].z, vraw[it].w) : make_uint4(0u, 0u, 0u, 0u), vd);
+        const int pl = it * 16 + slot;
+        const bool live = p0 + pl < ctx;
+        uint32_t* dst = &s_v[pl][4 * sub];
+        dst[0] = live ? vraw[it].x : 0u;
+        dst[1] = live ? vraw[it].y : 0u;
+        dst[2] = live ? vraw[it].z : 0u;
+        dst[3] = live ? vraw[it].w : 0u;
+    }
+    __syncthreads();
+
+    // pass 2: weighted sum of V rows on the matrix cores, D[head][dim] = sum over the chunk's
+    // positions in steps of 32, A = the softmax weights (row = head), B = the V rows (column = dim).
+    // Lane (mc, mb) supplies positions 32 s + 8 mb .. + 7 of head mc and of dim mc of the tile.  The
+    // weights are fp32 and the operands bf16: a weight enters as its bf16 rounding plus the bf16
+    // rounding of what that left over, two MFMAs per step (error 2^-17 relative instead of 2^-9).
+    // A wave takes two of the eight sixteen-dim tiles; nothing is left to add up across threads.
+    constexpr int KSTEPS = CHUNK / 32;
+    const uint16_t* sv16 = reinterpret_cast<const uint16_t*>(&s_v[0][0]);
+    f32x4v dacc[2];
+    dacc[0] = dacc[1] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            const float wgt = s_score[g][it * 16 + slot];
+    for (int ks = 0; ks < KSTEPS; ks++) {
+        const float4* prow = reinterpret_cast<const float4*>(&s_score[q_head][32 * ks + 8 * mb]);
+        const float4 pa = prow[0];
+        const float4 pb = prow[1];
+        const float pw[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
+        uint32_t hi[4], lo[4];
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc[g][i] = __builtin_fmaf(wgt, vd[i], acc[g][i]);
+        for (int j = 0; j < 4; j++) {
+            const float w0 = q_live ? pw[2 * j] : 0.0f;
+            const float w1 = q_live ? pw[2 * j + 1] : 0.0f;
+            hi[j] = f32x2_to_bf16x2(w0, w1);
+            lo[j] = f32x2_to_bf16x2(w0 - __uint_as_float(hi[j] << 16), w1 - __uint_as_float(hi[j] & 0xffff0000u));
+        }
+        const bf16x8 a_hi = as_bf16x8(hi[0], hi[1], hi[2], hi[3]);
+        const bf16x8 a_lo = as_bf16x8(lo[0], lo[1], lo[2], lo[3]);
+#pragma unroll
+        for (int n = 0; n < 2; n++) {
+            const int col = 16 * (2 * wave + n) + mc;  // dim
+            const uint16_t* vcol = sv16 + static_cast<size_t>(32 * ks + 8 * mb) * (2 * kVRow) + col;
+            uint32_t vw[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t even = vcol[(2 * j) * (2 * kVRow)];
+                const uint32_t odd = vcol[(2 * j + 1) * (2 * kVRow)];
+                vw[j] = even | (odd << 16);
+            }
+            const bf16x8 b_op = as_bf16x8(vw[0], vw[1], vw[2], vw[3]);
+            dacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_op, dacc[n], 0, 0, 0);
+            dacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b_op, dacc[n], 0, 0, 0);
         }
     }
-    // the sixteen position slots meet in LDS, at most four heads at a time
-    constexpr int GH = G < kAccHeads ? G : kAccHeads;
+    // the lane holds heads 4 mb .. 4 mb + 3 of dim `col`
 #pragma unroll
-    for (int g0 = 0; g0 < G; g0 += GH) {
-        if (g0 > 0) __syncthreads();
+    for (int n = 0; n < 2; n++) {
+        const int col = 16 * (2 * wave + n) + mc;
 #pragma unroll
-        for (int g = 0; g < GH; g++) {
-            float4* dst = reinterpret_cast<float4*>(&s_acc[slot][g][8 * sub]);
-            dst[0] = make_float4(acc[g0 + g][0], acc[g0 + g][1], acc[g0 + g][2], acc[g0 + g][3]);
-            dst[1] = make_float4(acc[g0 + g][4], acc[g0 + g][5], acc[g0 + g][6], acc[g0 + g][7]);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int o = tid; o < GH * kHeadDim; o += kAttnThreads) {
-            const int g = o / kHeadDim;
-            const int d = o % kHeadDim;
-            float part[kAttnSlots];
-#pragma unroll
-            for (int sl = 0; sl < kAttnSlots; sl++) part[sl] = s_acc[sl][g][d];
-            float sum = 0.0f;
-#pragma unroll
-            for (int sl = 0; sl < kAttnSlots; sl++) sum += part[sl];
-            out_base[g0 * kHeadDim + o] = sum;
+        for (int v = 0; v < 4; v++) {
+            const int head = 4 * mb + v;
+            if (head < G) out_base[head * kHeadDim + col] = dacc[n][v];
         }
     }
 }
