@@ -139,6 +139,18 @@ def test_ragged_and_small_shapes(capi, torch, oracle, K, N, G):
     check_against_oracle(oracle, p, y)
 
 
+@pytest.mark.parametrize("M", [6, 9, 16])
+@pytest.mark.parametrize("K,N,G", [(1024, 1008, 128), (512, 272, 128), (2048, 48, 64), (256, 16, 128),
+                                   (1536, 784, 256), (384, 264, 128), (8192, 512, 128)])
+def test_ragged_shapes_with_many_rows(capi, torch, oracle, M, K, N, G):
+    """Five to sixteen activation rows on column counts that end inside a tile (and, for the MFMA kernel's
+    two-column read-back, inside a pair of threads), on K that one workgroup covers, and on N that only
+    the vector kernel takes (not a multiple of sixteen)."""
+    p = synth.make_awq_problem(f"ragged_rows_{M}_{K}x{N}", M, K, N, group=G)
+    y, _ = run_awq(capi, torch, p)
+    check_against_oracle(oracle, p, y)
+
+
 def test_linearity_in_x_at_full_size(capi, torch):
     """y(a) + y(b) ~= y(a + b) at a full-size shape, a property that needs no oracle."""
     K, N = 4096, 12288
