@@ -27,6 +27,9 @@ inline int kernel_override() {
     return g_kernel_policy;
 }
 
+constexpr int kComputeUnits = 256;  // MI355X
+constexpr int kExchangeRows = 8;    // what a K tile's share of the split-K exchange costs, in rows of K streamed
+
 inline bool is_pow2(int v) {
     return v > 0 && (v & (v - 1)) == 0;
 }
@@ -59,29 +62,37 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
     p.coltiles = (N / 8 + kWC - 1) / kWC;
     p.mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
     p.mtiles = (M + p.mb - 1) / p.mb;
-    // Eight waves of sixteen rows per lane (256 rows of K per workgroup) measured best or within
-    // noise of best on every Qwen3 projection shape; shorter K takes fewer waves so that no
-    // workgroup is mostly idle.
+    // Three shapes of workgroup: eight waves of sixteen rows per lane (256 rows of K), eight waves of
+    // 32 rows per lane (512 rows, half the partial sums to exchange) and twelve waves of sixteen
+    // rows (384 rows).  What a launch costs, in rows of K streamed by the busiest compute unit, is
+    // the number of workgroups that compute unit gets (all of them resident together or not) times
+    // the rows of a workgroup, plus about eight rows' worth per K tile for the exchange.  Measured,
+    // us per launch at M = 1 (256 / 512 / 384 rows): q 4096->4096 5.7 / 6.2 / -, gate 4096->12288
+    // 8.6 / 9.3 / -, q|k|v 4096->6144 6.8 / 6.6 / -, gate|up 4096->24576 15.7 / 13.8 / -, down
+    // 12288->4096 10.0 / - / 9.1, 32B-shaped q|k|v 5120->10240 10.6 / 9.8 / -, o 8192->5120
+    // 9.1 / 9.3 / -: the minimum of that cost picks the faster one every time.
+    // Twelve waves: one activation row, plain or SwiGLU input, plain or residual output only (the
+    // other prologues and epilogues are laid out for 4 or 8 waves).  Shorter K than 256 takes fewer
+    // waves so that no workgroup is mostly idle.
     p.rt = 16;
     p.waves = 8;
-    // Matrices large enough to keep three workgroups per compute unit busy even so take 32 rows per
-    // lane (512 rows of K per workgroup): all workgroups are resident at once and half as many
-    // partial sums are exchanged.  Measured on the fused gate/up shape (4096 -> 24576): 15.7 -> 13.8 us.
-    constexpr int kRowsLong = 8 * kSlotsPerWave * 32;
-    if (allow_long_rows && K % kRowsLong == 0 && static_cast<long>(p.coltiles) * (K / kRowsLong) >= 768) {
-        p.rt = 32;
-        p.ktiles = K / kRowsLong;
-        return p;
-    }
-    // Long K on few column tiles (the 8B down projection, 12288 -> 4096): twelve waves, 384 rows per
-    // workgroup, give two workgroups of 768 threads per compute unit instead of three of 512 and 32
-    // K tiles to exchange instead of 48 (9.98 -> 9.05 us).  One activation row, plain or SwiGLU
-    // input, plain or residual output: the other prologues and epilogues are laid out for 4 or 8 waves.
-    constexpr int kRows12 = 12 * kSlotsPerWave * 16;
-    if (allow_12_waves && M == 1 && K % kRows12 == 0 && K / 256 >= 40 &&
-        static_cast<long>(p.coltiles) * (K / kRows12) >= 512) {
-        p.waves = 12;
-        p.ktiles = K / kRows12;
+    if (K >= rows_per_block(8, 16)) {
+        const struct { int waves, rt; bool allowed; } shapes[3] = {
+            {8, 16, true}, {8, 32, allow_long_rows}, {12, 16, allow_12_waves && M == 1}};
+        long best = -1;
+        for (const auto& c : shapes) {
+            const int rows = rows_per_block(c.waves, c.rt);
+            if (!c.allowed || (c.waves != 8 || c.rt != 16) && K % rows != 0) continue;
+            const long kt = (K + rows - 1) / rows;
+            const long blocks = static_cast<long>(p.coltiles) * p.mtiles * kt;
+            const long cost = (blocks + kComputeUnits - 1) / kComputeUnits * rows + kExchangeRows * kt;
+            if (best < 0 || cost < best) {
+                best = cost;
+                p.waves = c.waves;
+                p.rt = c.rt;
+                p.ktiles = static_cast<int>(kt);
+            }
+        }
         return p;
     }
     while (p.waves > 4 && rows_per_block(p.waves, p.rt) > K) p.waves /= 2;
