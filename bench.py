@@ -34,7 +34,7 @@ METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
 # HBM bytes per launch of the dominant kernel (average over the seven launches of a step) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
 # reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).
-TRAFFIC_BYTES_PER_LAUNCH = 15358600
+TRAFFIC_BYTES_PER_LAUNCH = 15288300
 
 
 def parse_args():
