@@ -243,27 +243,31 @@ def main():
                                          "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
                                          "bytes": b}
 
-        # the two launches a decode step fuses along N, same cold-weight protocol
-        fused_shapes = {"qkv fused": (4096, 6144), "gate+up fused": (4096, 24576)}
-        fsets = [WeightSet(torch, fused_shapes, group, gen) for _ in range(WEIGHT_SETS)]
-        for n, (K, N) in fused_shapes.items():
+        # The launches a decode step fuses along N, and the launches of the Qwen3-32B-shaped step: same
+        # cold-weight protocol, one shape at a time (the largest is 131 MB per copy).
+        more_shapes = {"qkv fused": (4096, 6144), "gate+up fused": (4096, 24576),
+                       "32B qkv fused": (5120, 10240), "32B o_proj": (8192, 5120),
+                       "32B gate+up fused": (5120, 51200), "32B down_proj": (25600, 5120)}
+        for n, (K, N) in more_shapes.items():
+            fsets = [WeightSet(torch, {n: (K, N)}, group, gen) for _ in range(WEIGHT_SETS)]
             b = synth.awq_gemv_bytes(1, K, N)
+            xf = xs[K] if K in xs else torch.randn((1, K), device="cuda", generator=gen).bfloat16()
             yf = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
             wsf = capi.make_workspace(1, K, N)
             reps = 240 // WEIGHT_SETS * WEIGHT_SETS
 
-            def launch_f(first, count, n=n, yf=yf, wsf=wsf, K=K):
+            def launch_f(first, count, n=n, xf=xf, yf=yf, wsf=wsf, fsets=fsets):
                 for s in range(first, first + count):
                     qw, sc, qz = fsets[s % WEIGHT_SETS].t[n]
-                    capi.gemv_awq_bf16(xs[K], qw, sc, qz, yf, group, wsf)
+                    capi.gemv_awq_bf16(xf, qw, sc, qz, yf, group, wsf)
 
             sec = timed_region(torch, launch_f, reps, WEIGHT_SETS, args.eager, WEIGHT_SETS)
             us = sec / reps * 1e6
             per_shape[f"{n} {K}x{N}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
                                          "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
                                          "bytes": b}
-        del fsets
-        torch.cuda.empty_cache()
+            del fsets, launch_f
+            torch.cuda.empty_cache()
 
     small_batch = None
     if not args.no_small_batch:
