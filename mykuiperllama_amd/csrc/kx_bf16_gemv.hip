@@ -1,8 +1,10 @@
 // BF16 GEMV fallback for gfx950: y[m,n] = sum_k x[m,k] * W[n,k], W bf16 row-major [N, K].
 //
-// One wave per output row: the 64 lanes walk the row in 16-byte pieces (eight bf16 each), pairs
-// along K go through the packed bf16 dot instruction with an fp32 accumulator, and the lanes
-// meet in a butterfly at the end.  Rows are contiguous, so every load is a full 1 KiB per wave.
+// One or two activation rows: one wave per output row, the 64 lanes walk the row in 16-byte pieces
+// (eight bf16 each), pairs along K go through the packed bf16 dot instruction with an fp32
+// accumulator, and the lanes meet in a wave-wide sum at the end.  Rows are contiguous, so every load
+// is a full 1 KiB per wave.  Three to sixteen rows: matrix cores, sixteen output rows per workgroup
+// (second kernel below).
 #include "kx_common.h"
 
 namespace kx {
@@ -94,6 +96,70 @@ __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
     }
 }
 
+// Three to sixteen activation rows: matrix cores, one pass over W whatever M is.
+// v_mfma_f32_16x16x32_bf16 with A = the activations (row m = lane % 16, zero rows past M) and
+// B = sixteen rows of W (column n = lane % 16): lane (c, b) supplies x[c][32 s + 8 b .. + 7] and
+// W[n0 + c][32 s + 8 b .. + 7], sixteen contiguous bytes each, and receives y[4 b + v][n0 + c].
+// A workgroup owns sixteen output columns; its four waves take the 32-element steps of K in turn
+// (step s goes to wave s % 4) in sweeps of kMfmaUnroll steps with all loads of a sweep in flight
+// together, and meet in LDS.  Addresses are clamped, what lies past K or M is zeroed in both operands.
+constexpr int kMfmaWaves = 4;
+constexpr int kMfmaUnroll = 8;
+
+__global__ __launch_bounds__(kMfmaWaves * kWave) void bf16_gemv_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y, int M, int K, int N) {
+    __shared__ float red[kMfmaWaves][4][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int c = lane % 16;
+    const int b = lane / 16;
+    const int n0 = blockIdx.x * 16;
+    const int n_ld = n0 + c < N ? n0 + c : N - 1;
+    const int m_ld = c < M ? c : M - 1;
+    const uint16_t* wrow = w + static_cast<size_t>(n_ld) * K;
+    const uint16_t* xrow = x + static_cast<size_t>(m_ld) * K;
+    const bool row_live = c < M;
+    const int k_last = K - 8;  // K is a multiple of eight
+
+    f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int kSweep = 32 * kMfmaWaves * kMfmaUnroll;  // elements of K a workgroup covers per sweep
+    for (int k0 = 32 * wave; k0 < K; k0 += kSweep) {
+        u32x4 wv[kMfmaUnroll], xv[kMfmaUnroll];
+#pragma unroll
+        for (int u = 0; u < kMfmaUnroll; u++) {
+            const int k = k0 + 32 * kMfmaWaves * u + 8 * b;
+            wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (k < K ? k : k_last)));
+        }
+#pragma unroll
+        for (int u = 0; u < kMfmaUnroll; u++) {
+            const int k = k0 + 32 * kMfmaWaves * u + 8 * b;
+            xv[u] = *reinterpret_cast<const u32x4*>(xrow + (k < K ? k : k_last));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // every load of the sweep is out before the first is waited for
+#pragma unroll
+        for (int u = 0; u < kMfmaUnroll; u++) {
+            const bool live = k0 + 32 * kMfmaWaves * u + 8 * b < K;
+            const bool a_live = live && row_live;
+            const bf16x8 a_op = as_bf16x8(a_live ? xv[u].x : 0u, a_live ? xv[u].y : 0u, a_live ? xv[u].z : 0u,
+                                          a_live ? xv[u].w : 0u);
+            const bf16x8 b_op = as_bf16x8(live ? wv[u].x : 0u, live ? wv[u].y : 0u, live ? wv[u].z : 0u,
+                                          live ? wv[u].w : 0u);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, b_op, acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) red[wave][v][lane] = acc[v];
+    __syncthreads();
+    if (wave == 0 && n0 + c < N) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int m = 4 * b + v;
+            const float sum = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
+            if (m < M) y[static_cast<size_t>(m) * N + n0 + c] = f32_to_bf16(sum);
+        }
+    }
+}
+
 }  // namespace
 }  // namespace kx
 
@@ -108,19 +174,20 @@ extern "C" int kx_gemv_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, i
         return KX_ERR_ALIGNMENT;
     }
     hipStream_t s = kx::as_stream(stream);
-    dim3 grid((N + kx::kRowsPerBlock - 1) / kx::kRowsPerBlock);
-    dim3 block(kx::kRowsPerBlock * kx::kWave);
-    for (int m0 = 0; m0 < M; m0 += 4) {
-        const int mb = M - m0 >= 4 ? 4 : (M - m0 >= 2 ? 2 : 1);
-        if (mb == 4) {
-            hipLaunchKernelGGL((kx::bf16_gemv_kernel<4>), grid, block, 0, s, x, w, y, M, K, N, m0);
-        } else if (mb == 2) {
-            hipLaunchKernelGGL((kx::bf16_gemv_kernel<2>), grid, block, 0, s, x, w, y, M, K, N, m0);
-            m0 -= 2;  // step of 4 below; a 2-row pass advances by 2
-        } else {
-            hipLaunchKernelGGL((kx::bf16_gemv_kernel<1>), grid, block, 0, s, x, w, y, M, K, N, m0);
-            m0 -= 3;
-        }
+    if (M >= 3) {
+        // One pass on the matrix cores (lm_head 151936 x 4096: 270 us at M = 3..5, 300 at 8, 370 at 16;
+        // the vector kernel, whose every wave reads the activation rows for itself, needs 310 us
+        // for four rows and would need a pass over W per four rows beyond that).
+        hipLaunchKernelGGL(kx::bf16_gemv_mfma_kernel, dim3((N + 15) / 16), dim3(kx::kMfmaWaves * kx::kWave), 0, s, x, w,
+                           y, M, K, N);
+        return kx::launch_status();
+    }
+    const dim3 grid((N + kx::kRowsPerBlock - 1) / kx::kRowsPerBlock);
+    const dim3 block(kx::kRowsPerBlock * kx::kWave);
+    if (M == 1) {
+        hipLaunchKernelGGL((kx::bf16_gemv_kernel<1>), grid, block, 0, s, x, w, y, M, K, N, 0);
+    } else {
+        hipLaunchKernelGGL((kx::bf16_gemv_kernel<2>), grid, block, 0, s, x, w, y, M, K, N, 0);
     }
     return kx::launch_status();
 }
