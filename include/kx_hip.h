@@ -252,8 +252,8 @@ int kx_awq_dequant_bf16(const int32_t* qweight, const uint16_t* scales, const in
  *                         (bf16 [cache_positions][n_kv_heads][128]; a position outside
  *                         0 .. cache_positions-1 writes no cache row).  head_dim must be 128.
  *   kx_attn_decode_bf16   GQA attention of one query position against cache rows 0 .. *pos:
- *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv in
- *                         {1,2,4,8}; split over the context in chunks, merged by log-sum-exp.
+ *                         out[h,:] = softmax(q[h,:] . K[:,h/G,:] / sqrt(128)) V[:,h/G,:], G = n_q/n_kv
+ *                         between 1 and 16; split over the context in chunks, merged by log-sum-exp.
  *                         `max_positions` (<= 65536) fixes the launch shape (a captured graph can be
  *                         replayed while *pos advances up to max_positions - 1) and the chunk size:
  *                         64 positions up to max_positions = 5120, 128 beyond.

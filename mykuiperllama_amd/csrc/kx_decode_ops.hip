@@ -129,16 +129,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __res
 // Stage 2: one wave per query head merges the chunks by log-sum-exp and writes bf16.
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnThreads = 256;
-constexpr int kMaxGroup = 8;  // query heads per KV head this kernel is instantiated for
+constexpr int kMaxGroup = 16;  // query heads per KV head: the rows of one MFMA tile
 
-template <int G, int CHUNK>
+template <int CHUNK>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
-    float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, const int32_t* __restrict__ pos_ptr,
+    float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, int G, const int32_t* __restrict__ pos_ptr,
     int nchunks, int max_positions, float scale) {
     // Scores, then softmax weights, per head; rows padded so that the sixteen-byte reads of the
     // second pass (one row per lane) do not all start on the same bank.
-    __shared__ __attribute__((aligned(16))) float s_score[G][CHUNK + 4];
+    __shared__ __attribute__((aligned(16))) float s_score[kMaxGroup][CHUNK + 4];
     // The chunk's V rows, row-major, one dword of padding per row: the second pass reads them
     // transposed (eight positions of one dim per lane), and with 65 dwords per row the four blocks of
     // eight positions that a read instruction touches fall on different banks.
@@ -321,10 +321,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
 
 constexpr int kMergeThreads = kHeadDim * kMergeParts;
 
-template <int G>
 __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float* __restrict__ part_out,
                                                                     const float* __restrict__ part_ml,
-                                                                    uint16_t* __restrict__ out, int nchunks) {
+                                                                    uint16_t* __restrict__ out, int G, int nchunks) {
     extern __shared__ float s_factor[];  // nchunks rescaling factors exp(m_c - m)
     __shared__ float s_norm;
     __shared__ float s_part[kMergeParts][kHeadDim];
@@ -543,7 +542,7 @@ int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_ca
         return KX_ERR_BAD_SHAPE;
     }
     const int G = n_q_heads / n_kv_heads;
-    if (G != 1 && G != 2 && G != 4 && G != 8) return KX_ERR_BAD_SHAPE;
+    if (G > kx::kMaxGroup) return KX_ERR_BAD_SHAPE;
     if (workspace_bytes < kx_attn_decode_workspace_bytes(n_q_heads, head_dim, max_positions)) return KX_ERR_WORKSPACE;
     if (!kx::aligned16(q) || !kx::aligned16(k_cache) || !kx::aligned16(v_cache) || !kx::aligned16(workspace)) {
         return KX_ERR_ALIGNMENT;
@@ -556,22 +555,17 @@ int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_ca
     const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
     hipStream_t s = kx::as_stream(stream);
     dim3 grid1(nchunks, n_kv_heads);
-#define KX_ATTN(GG)                                                                                             \
-    if (long_chunks) {                                                                                          \
-        hipLaunchKernelGGL((kx::attn_decode_stage1<GG, kx::kAttnChunkLong>), grid1, dim3(kx::kAttnThreads), 0,  \
-                           s, q, k_cache, v_cache, part_out, part_ml, n_kv_heads, pos, nchunks, max_positions,  \
-                           scale);                                                                              \
-    } else {                                                                                                    \
-        hipLaunchKernelGGL((kx::attn_decode_stage1<GG, kx::kAttnChunkShort>), grid1, dim3(kx::kAttnThreads), 0, \
-                           s, q, k_cache, v_cache, part_out, part_ml, n_kv_heads, pos, nchunks, max_positions,  \
-                           scale);                                                                              \
-    }                                                                                                           \
-    if (out) {                                                                                                  \
-        hipLaunchKernelGGL((kx::attn_decode_stage2<GG>), dim3(n_q_heads), dim3(kx::kMergeThreads),              \
-                           nchunks * sizeof(float), s, part_out, part_ml, out, nchunks);                        \
+    if (long_chunks) {
+        hipLaunchKernelGGL((kx::attn_decode_stage1<kx::kAttnChunkLong>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache,
+                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale);
+    } else {
+        hipLaunchKernelGGL((kx::attn_decode_stage1<kx::kAttnChunkShort>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache,
+                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale);
     }
-    if (G == 1) { KX_ATTN(1) } else if (G == 2) { KX_ATTN(2) } else if (G == 4) { KX_ATTN(4) } else { KX_ATTN(8) }
-#undef KX_ATTN
+    if (out) {
+        hipLaunchKernelGGL(kx::attn_decode_stage2, dim3(n_q_heads), dim3(kx::kMergeThreads), nchunks * sizeof(float), s,
+                           part_out, part_ml, out, G, nchunks);
+    }
     return kx::launch_status();
 }
 }  // namespace

@@ -1,6 +1,6 @@
 // MultiHeadAttention: grouped-query attention of one query position against cache rows 0 .. pos
 // (the LayerMHA slot, kuiper/include/op/layer.h:15; the reference's mha.h is an empty namespace).
-// out[h, :] = softmax(q[h, :] . K[:, h / G, :] / sqrt(128)) V[:, h / G, :], G = n_q / n_kv in {1, 2, 4, 8}.
+// out[h, :] = softmax(q[h, :] . K[:, h / G, :] / sqrt(128)) V[:, h / G, :], G = n_q / n_kv between 1 and 16.
 //   input 0    q bf16 [n_q * 128]
 //   input 1    pos int32 [1] on the layer's device
 //   input 2    k_cache bf16 [max_positions, n_kv, 128]     input 3   v_cache, same shape

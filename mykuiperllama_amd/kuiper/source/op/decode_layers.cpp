@@ -204,15 +204,15 @@ base::Status MultiHeadAttention::check() const {
         return base::error::invalid_argument("The head counts of the mha layer are invalid.");
     }
     const int32_t g = n_q_ / n_kv_;
-    if (g != 1 && g != 2 && g != 4 && g != 8) {
-        return base::error::invalid_argument("The mha layer serves 1, 2, 4 or 8 query heads per key/value head.");
+    if (g > 16) {
+        return base::error::invalid_argument("The mha layer serves up to 16 query heads per key/value head.");
     }
     KX_RETURN_IF_BAD(expect(get_input(0), base::DataType::DataTypeBf16, static_cast<size_t>(n_q_) * kHeadDim, "query"));
     KX_RETURN_IF_BAD(expect(get_input(1), base::DataType::DataTypeInt32, 1, "pos"));
     const tensor::Tensor& kc = get_input(2);
     if (kc.is_empty() || kc.dims_size() != 3 || kc.get_dim(1) != n_kv_ || kc.get_dim(2) != kHeadDim ||
-        kc.get_dim(0) > 32768) {
-        return base::error::invalid_argument("The key cache must be [max_positions <= 32768, n_kv_heads, 128].");
+        kc.get_dim(0) > 65536) {
+        return base::error::invalid_argument("The key cache must be [max_positions <= 65536, n_kv_heads, 128].");
     }
     KX_RETURN_IF_BAD(expect(kc, base::DataType::DataTypeBf16, kc.size(), "key cache"));
     KX_RETURN_IF_BAD(expect(get_input(3), base::DataType::DataTypeBf16, kc.size(), "value cache"));

@@ -138,7 +138,7 @@ def test_cache_append_skips_positions_outside_the_cache(capi, torch, pos):
     assert torch.isfinite(q_out.float()).all()
 
 
-@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (8, 4), (4, 4)])
+@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (8, 4), (4, 4), (40, 8), (12, 4), (16, 1)])
 @pytest.mark.parametrize("ctx,max_pos", [(1, 4224), (5, 4224), (128, 4224), (129, 4224), (1000, 4224), (4097, 4224),
                                          # caches past 5120 positions are walked in chunks of 128
                                          (1, 5121), (127, 8320), (128, 8320), (129, 8320), (8193, 8320),

@@ -251,6 +251,8 @@ MERGE_CASES = [
     (8, 2, 5000, 5121, 512, 128),     # just past the switch to chunks of 128
     (64, 8, 1000, 1100, 5120, 128),   # eight query heads per KV head
     (4, 2, 37, 48, 512, 128),
+    (40, 8, 700, 768, 1024, 128),     # Qwen3-14B's grouping: five query heads per KV head
+    (6, 2, 300, 6000, 264, 64),       # three per KV head, chunks of 128 positions
     (2, 1, 100, 128, 264, 32),        # K = 256, ragged N
     (1, 1, 5, 64, 64, 32),            # K = 128: four waves, one head
     (4, 4, 127, 128, 256, 64),        # no grouping, context ends on a chunk boundary
