@@ -71,6 +71,9 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
     // 8.6 / 9.3 / -, q|k|v 4096->6144 6.8 / 6.6 / -, gate|up 4096->24576 15.7 / 13.8 / -, down
     // 12288->4096 10.0 / - / 9.1, 32B-shaped q|k|v 5120->10240 10.6 / 9.8 / -, o 8192->5120
     // 9.1 / 9.3 / -: the minimum of that cost picks the faster one every time.
+    // (Twelve waves of 32 rows, 768 rows per workgroup and one workgroup per compute unit on down
+    // 12288->4096, are faster still on the plain launch, 9.0 -> 8.6 us, but slower with the SwiGLU
+    // prologue of the decode step, whose latency then has no second workgroup to hide behind.)
     // Twelve waves: one activation row, plain or SwiGLU input, plain or residual output only (the
     // other prologues and epilogues are laid out for 4 or 8 waves).  Shorter K than 256 takes fewer
     // waves so that no workgroup is mostly idle.
