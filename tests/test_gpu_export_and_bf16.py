@@ -90,6 +90,23 @@ def test_bf16_gemv_matches_oracle(capi, torch, oracle, M, K, N):
     assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 16])
+@pytest.mark.parametrize("K,N", [(8, 1), (40, 15), (1000, 17), (4104, 1001), (72, 64)])
+def test_bf16_gemv_ragged_shapes(capi, torch, oracle, M, K, N):
+    """K that is a multiple of eight but not of a sweep or of a 32-element MFMA step, N below and just past a
+    tile of sixteen rows, for the one-row, two-row and matrix-core kernels."""
+    p = synth.make_bf16_problem(f"bf16_ragged_{M}_{K}x{N}", M, K, N)
+    y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_bf16(H.to_dev_bf16(p["x"], torch), H.to_dev_bf16(p["w"], torch), y)
+    torch.cuda.synchronize()
+    ref64 = oracle.gemv_bf16_f64(p["x"], p["w"])
+    ref_rounded = H.bf16_to_f64(oracle.f32_to_bf16(ref64.astype(np.float32)))
+    got = H.bf16_to_f64(H.bf16_bits(y, torch))
+    assert np.isfinite(got).all()
+    assert H.rel_l2(got, ref_rounded) <= 1e-3
+    assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
+
+
 def test_bf16_gemv_one_hot_returns_the_weight_column_exactly(capi, torch):
     K, N = 1024, 512
     p = synth.make_bf16_problem("bf16_onehot", 1, K, N)
