@@ -160,6 +160,60 @@ def test_decode_steps_match_the_fp32_reference(torch, oracle, fused):
     assert agreed >= 1
 
 
+@pytest.mark.parametrize("fused", [True, "prologue", False])
+def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, oracle, fused):
+    """An independent implementation of the architecture: the installed `transformers` Qwen3 model (eager
+    attention, fp32, on the CPU) is given the dequantised weights and run over a token sequence in one pass;
+    the decode step here is fed the same tokens one by one from an empty KV cache.  This pins what the
+    in-file fp32 restatement could share a misreading with: where the norms sit, the rotate-half convention
+    and its frequencies, which query heads go with which KV head, the residual wiring and SwiGLU."""
+    from transformers import Qwen3Config, Qwen3ForCausalLM
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    layers_np, layers_ref, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
+    hf_cfg = Qwen3Config(vocab_size=cfg.vocab, hidden_size=cfg.hidden, intermediate_size=cfg.intermediate,
+                         num_hidden_layers=cfg.layers, num_attention_heads=cfg.n_q, num_key_value_heads=cfg.n_kv,
+                         head_dim=128, rms_norm_eps=cfg.eps, rope_theta=cfg.rope_theta, tie_word_embeddings=False,
+                         attention_bias=False, max_position_embeddings=MAXPOS, attn_implementation="eager")
+    hf = Qwen3ForCausalLM(hf_cfg).eval().float()
+    sd = {"model.embed_tokens.weight": embed.float(), "model.norm.weight": final_norm.float(),
+          "lm_head.weight": lm_head.float()}
+    for li, (w, n) in enumerate(layers_ref):
+        pre = f"model.layers.{li}."
+        for name in ("q", "k", "v", "o"):
+            sd[pre + f"self_attn.{name}_proj.weight"] = w[name].T.contiguous()  # Linear keeps [out, in]
+        for name in ("gate", "up", "down"):
+            sd[pre + f"mlp.{name}_proj.weight"] = w[name].T.contiguous()
+        sd[pre + "self_attn.q_norm.weight"] = n["q_norm"].float()
+        sd[pre + "self_attn.k_norm.weight"] = n["k_norm"].float()
+        sd[pre + "input_layernorm.weight"] = n["in_norm"].float()
+        sd[pre + "post_attention_layernorm.weight"] = n["post_norm"].float()
+    missing, unexpected = hf.load_state_dict(sd, strict=False)
+    assert not unexpected and all("rotary" in m or "inv_freq" in m for m in missing), (missing, unexpected)
+
+    tokens = [17, 3, 900, 41, 512, 7, 1023, 64, 5, 250, 77, 12]
+    with torch.no_grad():
+        hf_logits = hf(torch.tensor([tokens])).logits[0]  # [len, vocab], causal: row p sees tokens 0..p
+
+    model = decode.DecodeModel(cfg, MAXPOS, weights=to_model_weights(torch, layers_np, embed, lm_head, final_norm))
+    agreed = 0
+    for pos, token in enumerate(tokens):
+        model.set_input(token, pos)
+        model.step(fused=fused)
+        torch.cuda.synchronize()
+        got = model.logits[0].cpu().float()
+        ref = hf_logits[pos]
+        assert torch.isfinite(got).all()
+        # the GPU path stores bf16 after every operator, the library computes in fp32 throughout
+        err = ((got - ref).norm() / ref.norm()).item()
+        assert err <= 3e-2, f"position {pos}: logits relative L2 {err}"
+        top2 = ref.topk(2).values
+        if (top2[0] - top2[1]) > 0.05 * top2[0].abs():
+            assert int(model.next_token.item()) == int(ref.argmax())
+            agreed += 1
+    assert agreed >= 3
+
+
 def test_fused_and_separate_launches_give_the_same_step(torch):
     """SwiGLU and add+RMSNorm in the GEMV prologue change nothing, bit for bit."""
     from mykuiperllama_amd import decode
