@@ -160,8 +160,9 @@ def test_decode_steps_match_the_fp32_reference(torch, oracle, fused):
     assert agreed >= 1
 
 
-@pytest.mark.parametrize("fused", [True, "prologue", False])
-def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, oracle, fused):
+@pytest.mark.parametrize("fused,max_pos", [(True, MAXPOS), ("prologue", MAXPOS), (False, MAXPOS),
+                                           (True, 6000), (True, 10368)])  # chunks of 128; merge as its own launch
+def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, oracle, fused, max_pos):
     """An independent implementation of the architecture: the installed `transformers` Qwen3 model (eager
     attention, fp32, on the CPU) is given the dequantised weights and run over a token sequence in one pass;
     the decode step here is fed the same tokens one by one from an empty KV cache.  This pins what the
@@ -195,7 +196,7 @@ def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, 
     with torch.no_grad():
         hf_logits = hf(torch.tensor([tokens])).logits[0]  # [len, vocab], causal: row p sees tokens 0..p
 
-    model = decode.DecodeModel(cfg, MAXPOS, weights=to_model_weights(torch, layers_np, embed, lm_head, final_norm))
+    model = decode.DecodeModel(cfg, max_pos, weights=to_model_weights(torch, layers_np, embed, lm_head, final_norm))
     agreed = 0
     for pos, token in enumerate(tokens):
         model.set_input(token, pos)
