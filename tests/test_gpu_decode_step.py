@@ -160,9 +160,14 @@ def test_decode_steps_match_the_fp32_reference(torch, oracle, fused):
     assert agreed >= 1
 
 
-@pytest.mark.parametrize("fused,max_pos", [(True, MAXPOS), ("prologue", MAXPOS), (False, MAXPOS),
-                                           (True, 6000), (True, 10368)])  # chunks of 128; merge as its own launch
-def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, oracle, fused, max_pos):
+# a second head layout: five query heads per KV head (Qwen3-14B's grouping), ten heads of 128 on hidden 512
+CFG_G5 = dict(CFG, n_q=10, n_kv=2)
+
+
+@pytest.mark.parametrize("fused,max_pos,shape", [(True, MAXPOS, CFG), ("prologue", MAXPOS, CFG), (False, MAXPOS, CFG),
+                                                 (True, 6000, CFG), (True, 10368, CFG),  # chunks of 128; separate merge
+                                                 (True, MAXPOS, CFG_G5), (False, MAXPOS, CFG_G5)])
+def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, oracle, fused, max_pos, shape):
     """An independent implementation of the architecture: the installed `transformers` Qwen3 model (eager
     attention, fp32, on the CPU) is given the dequantised weights and run over a token sequence in one pass;
     the decode step here is fed the same tokens one by one from an empty KV cache.  This pins what the
@@ -170,7 +175,7 @@ def test_decode_from_an_empty_cache_matches_the_transformers_qwen3_model(torch, 
     and its frequencies, which query heads go with which KV head, the residual wiring and SwiGLU."""
     from transformers import Qwen3Config, Qwen3ForCausalLM
     from mykuiperllama_amd import decode
-    cfg = decode.ModelConfig(**CFG)
+    cfg = decode.ModelConfig(**shape)
     layers_np, layers_ref, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
     hf_cfg = Qwen3Config(vocab_size=cfg.vocab, hidden_size=cfg.hidden, intermediate_size=cfg.intermediate,
                          num_hidden_layers=cfg.layers, num_attention_heads=cfg.n_q, num_key_value_heads=cfg.n_kv,
