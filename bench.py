@@ -48,7 +48,8 @@ def parse_args():
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-small-batch", action="store_true", help="skip the M = 1..16 vector/MFMA kernel table")
     ap.add_argument("--no-decode", action="store_true", help="skip the Qwen3-8B decode-step measurement")
-    ap.add_argument("--decode-32b", action="store_true", help="also run the Qwen3-32B-shaped decode step")
+    ap.add_argument("--no-decode-32b", action="store_true", help="skip the Qwen3-32B-shaped decode step")
+    ap.add_argument("--decode-32b", action="store_true", help="kept for older command lines: the step runs by default")
     ap.add_argument("--decode-steps", type=int, default=60)
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection workload: one 256 MiB device copy (known traffic, for scaling the "
@@ -330,7 +331,7 @@ def main():
         d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager)
         out["decode_tok_s"] = d8["with_lm_head"]["tokens_per_s"]
         out["decode"] = {"qwen3-8b ctx4096": d8}
-        if args.decode_32b:
+        if not args.no_decode_32b:
             out["decode"]["qwen3-32b ctx8192"] = decode_benchmark(torch, "qwen3-32b", 8192, args.decode_steps, 8,
                                                                   args.eager)
     if not args.no_cpu_baseline:
