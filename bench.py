@@ -16,7 +16,7 @@ Prints one JSON line:  value = algorithmic bytes of a step / time of a step, in 
   per_shape     each projection shape on its own, cold weights, same event timing
   small_batch   configs[2]: M in {1, 2, 4, 8, 16} on three shapes, microseconds per launch of the
                 vector-ALU kernel and of the MFMA kernel (cold weights, same event timing)
-  decode        configs[3] (and configs[4] with --decode-32b): tokens/s of a full decode step
+  decode        configs[3] and configs[4]: tokens/s of a full decode step (Qwen3-8B, Qwen3-32B-shaped)
 """
 import argparse
 import json
