@@ -59,7 +59,8 @@ const char* kx_error_string(int code);
  *
  * A GEMV leaves the counters zeroed again, so one initialised workspace serves any number of
  * consecutive launches on ONE stream.  Launches that may overlap (different streams) need
- * separate workspaces.  The buffer must be 256-byte aligned.
+ * separate workspaces.  The buffer must be 256-byte aligned.  Shapes whose partial sums would
+ * take 4 GiB or more are rejected (KX_ERR_BAD_SHAPE); no Qwen3-sized projection comes near.
  * Reference counterpart: none (the reference has no split reduction); the allocator that
  * would provide the buffer is base::CUDADeviceAllocator, kuiper/source/base/alloc_cu.cpp:8-16.
  * ------------------------------------------------------------------------------------------ */
