@@ -10,7 +10,8 @@
 //   y_part[n] = s[g,n] * ( sum_r (16 + q[k0+r,n]) * x[k0+r]  -  (16 + z[g,n]) * sum_r x[k0+r] )
 //
 // A wave covers 32 consecutive word columns (128 contiguous bytes of each row, 256 output
-// columns) times two row slots; a workgroup stacks WAVES waves along K.  Row slots meet in LDS.
+// columns) times two row slots; a workgroup stacks WAVES waves along K.  The two row slots of a
+// wave meet through a lane exchange, the waves of a workgroup in LDS.
 // Workgroups that share a column tile meet in a caller-provided workspace: each stores its 256
 // partial sums, then bumps the tile's arrival counter; the workgroup that arrives last adds the
 // partials in a fixed order (bitwise reproducible) and writes y.  Thread t of a workgroup owns
