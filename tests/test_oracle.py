@@ -90,6 +90,14 @@ def test_unpack_known_answer_word(oracle):
         assert codes[0, col] == i
 
 
+def test_unpack_treats_the_sign_bit_as_payload(oracle):
+    # 0xFFFFFFFF is the int32 -1: eight codes of 15, the top nibble included.
+    assert oracle.awq_unpack(np.array([[-1]], np.int32)).tolist() == [[15] * 8]
+    assert oracle.awq_pack(np.full((1, 8), 15, np.uint8)).view(np.uint32).tolist() == [[0xFFFFFFFF]]
+    # 0x80000000: only nibble 7 (column ORDER[7] = 7) is set, to 8.
+    assert oracle.awq_unpack(np.array([[-2**31]], np.int32)).tolist() == [[0, 0, 0, 0, 0, 0, 0, 8]]
+
+
 def test_pack_every_position_and_code(oracle):
     for col in range(8):
         for code in range(16):
