@@ -24,6 +24,7 @@ KX_LIB = os.path.join(LIB_DIR, "libkx_hip.so")
 KUIPER_LIB = os.path.join(LIB_DIR, "libkuiper.so")
 KUIPER_TEST = os.path.join(LIB_DIR, "test_kuiper")
 SAFETENSORS_DUMP = os.path.join(LIB_DIR, "kx_safetensors_dump")
+QWEN3_DECODE = os.path.join(LIB_DIR, "kx_qwen3_decode")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU forms are switched off for all device code
@@ -57,6 +58,8 @@ def build_kuiper():
          ["-L", LIB_DIR, "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", KUIPER_LIB])
     _run([HIPCC, "--offload-arch=gfx950"] + COMMON + inc + [os.path.join(KUIPER, "app", "safetensors_dump.cpp")] +
          ["-L", LIB_DIR, "-lkuiper", "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", SAFETENSORS_DUMP])
+    _run([HIPCC, "--offload-arch=gfx950"] + COMMON + inc + [os.path.join(KUIPER, "app", "qwen3_decode.cpp")] +
+         ["-L", LIB_DIR, "-lkuiper", "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", QWEN3_DECODE])
     # C++ tests of the host API live under tests/cpp and link the CPU oracle as their checker
     tests = sorted(glob.glob(os.path.join(TESTS_CPP, "*.cpp")) + glob.glob(os.path.join(TESTS_CPP, "*.hip")))
     if tests:

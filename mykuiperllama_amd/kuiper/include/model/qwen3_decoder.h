@@ -1,0 +1,111 @@
+// Qwen3-style decoder, one token at a time (batch 1), on the GPU: INT4 AWQ projections, bf16 KV
+// cache, greedy sampling.  The reference lists kuiper/source/model/ in its build
+// (CMakeLists.txt:79) and the directory is absent; the layer slots of kuiper/include/op/layer.h:8-20
+// say which operators a model is made of.  This is the runner for them: weights attach through
+// MatmulLayer (model/safetensors.h), and a step is the launch sequence of include/kx_hip.h's fused
+// entry points, five or six launches per decoder layer:
+//
+//   x = embed[token]
+//   per layer:  q|k|v GEMV   (RMSNorm on the way in; per-head norm, rotation, cache append on the way out)
+//               attention    (partial results per chunk of the context)
+//               o GEMV       (merge of the chunks on the way in when the context allows; residual add out)
+//               gate|up GEMV (RMSNorm on the way in)
+//               down GEMV    (SwiGLU on the way in; residual add out)
+//   logits = lm_head RMSNorm(x);  next = argmax(logits)
+//
+// Token and position are read from device memory, so the whole step can be captured once in a HIP
+// graph and replayed for every token: capture() does that, step() then replays.
+#ifndef KUIPER_INCLUDE_MODEL_QWEN3_DECODER_H
+#define KUIPER_INCLUDE_MODEL_QWEN3_DECODER_H
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "base/base.h"
+#include "base/cuda_config.h"
+#include "model/safetensors.h"
+#include "op/matmul.h"
+#include "tensor/tensor.h"
+
+namespace model {
+
+struct Qwen3Config {
+    int32_t layers = 0;
+    int32_t hidden = 0;
+    int32_t intermediate = 0;
+    int32_t n_q_heads = 0;
+    int32_t n_kv_heads = 0;
+    int32_t vocab = 0;
+    int32_t head_dim = 128;  // the only head size the kernels are built for
+    int32_t group_size = 128;
+    float rope_theta = 1e6f;
+    float rms_eps = 1e-6f;
+
+    int32_t qkv_out() const { return (n_q_heads + 2 * n_kv_heads) * head_dim; }
+
+    // Reads the sizes off the tensors of a checkpoint with Hugging Face's Qwen3 names
+    // (model.layers.<i>.self_attn.q_proj.qweight ...).  rope_theta / rms_norm_eps / group_size are
+    // taken from the file's metadata when present.
+    static base::Status from_file(const SafetensorsFile& file, Qwen3Config& config);
+};
+
+class Qwen3Decoder {
+public:
+    // Allocates caches and scratch rows for max_positions positions.  The decoder runs on a stream
+    // of its own (graph capture needs one that is not the default stream).
+    Qwen3Decoder(const Qwen3Config& config, int32_t max_positions);
+    ~Qwen3Decoder();
+    Qwen3Decoder(const Qwen3Decoder&) = delete;
+    Qwen3Decoder& operator=(const Qwen3Decoder&) = delete;
+
+    // Copies the weights to the GPU: q|k|v and gate|up side by side along N, norms, embedding,
+    // lm_head (the embedding table when the file has no lm_head.weight).  BF16 or F16 on file for the
+    // unquantised tensors (F16 is rounded to bf16).
+    base::Status load(const SafetensorsFile& file);
+
+    // One token at position pos (0 <= pos < max_positions): appends its key and value to the caches
+    // and returns the most likely next token.  Synchronises the decoder's stream.
+    base::Status step(int32_t token, int32_t pos, int32_t* next_token);
+
+    // Records the step in a HIP graph; later step() calls replay it.
+    base::Status capture();
+    bool captured() const { return graph_exec_ != nullptr; }
+
+    // bf16 logits of the last step, copied to the host.
+    std::vector<uint16_t> logits() const;
+
+    const Qwen3Config& config() const { return config_; }
+    int32_t max_positions() const { return max_positions_; }
+    int32_t launches_per_step() const;
+    hipStream_t stream() const { return stream_->stream(); }
+
+private:
+    struct LayerWeights {
+        std::unique_ptr<op::MatmulLayer> qkv, o, gate_up, down;
+        tensor::Tensor input_norm, post_norm, q_norm, k_norm;
+        tensor::Tensor k_cache, v_cache;
+    };
+
+    int enqueue_step();  // 0 or the first failing entry point's return code
+
+    Qwen3Config config_;
+    int32_t max_positions_ = 0;
+    bool merge_in_o_ = false;
+    bool loaded_ = false;
+    std::shared_ptr<kernel::CudaConfig> stream_;
+    std::vector<LayerWeights> layers_;
+    tensor::Tensor embed_, final_norm_;
+    std::unique_ptr<op::MatmulLayer> lm_head_;
+    tensor::Tensor x_, h_, q_, attn_, gate_up_, logits_, sumsq_;
+    tensor::Tensor gemv_workspace_, attn_workspace_;
+    tensor::Tensor io_;           // device: token, position, next token (int32 each)
+    int32_t* host_io_ = nullptr;  // pinned mirror of io_
+    hipGraph_t graph_ = nullptr;
+    hipGraphExec_t graph_exec_ = nullptr;
+};
+
+}  // namespace model
+
+#endif  // KUIPER_INCLUDE_MODEL_QWEN3_DECODER_H

@@ -78,6 +78,11 @@ base::Status load_awq_linear_fused(const SafetensorsFile& file, const std::vecto
 // Attaches a BF16 [N, K] tensor to an unquantised MatmulLayer.
 base::Status load_bf16_linear(const SafetensorsFile& file, const std::string& name, op::MatmulLayer& layer);
 
+// A tensor of the given shape as bf16 in memory of `device` (norm gains, embedding table).  BF16 on
+// file is copied; F16 and F32 are rounded to bf16 (nearest, ties to even) on the way.
+base::Status load_bf16_tensor(const SafetensorsFile& file, const std::string& name, const std::vector<int32_t>& dims,
+                              base::DeviceType device, tensor::Tensor& out);
+
 }  // namespace model
 
 #endif  // KUIPER_INCLUDE_MODEL_SAFETENSORS_H

@@ -9,6 +9,7 @@
 #include <cstring>
 
 #include "base/alloc.h"
+#include "kernel/cpu/bf16.h"
 #include "tensor/tensor.h"
 
 namespace model {
@@ -534,6 +535,32 @@ base::Status load_bf16_linear(const SafetensorsFile& file, const std::string& na
     tensor::Tensor weight = device_tensor(base::DataType::DataTypeBf16, {layer.dim0(), layer.dim1()},
                                           layer.device_type(), file.data(*w), w->byte_size());
     return layer.set_weight(0, weight);
+}
+
+base::Status load_bf16_tensor(const SafetensorsFile& file, const std::string& name, const std::vector<int32_t>& dims,
+                              base::DeviceType device, tensor::Tensor& out) {
+    if (!file.is_open()) return base::error::invalid_argument("safetensors: the file is not open");
+    const TensorEntry* e = file.find(name);
+    if (!e) return base::error::path_not_valid("safetensors: " + name + " is not in the file");
+    bool same = e->shape.size() == dims.size();
+    for (size_t i = 0; same && i < dims.size(); i++) same = e->shape[i] == dims[i];
+    if (!same) return bad_file(name + ": shape differs from what the model expects");
+    const size_t count = static_cast<size_t>(e->element_count());
+    if (e->dtype == "BF16") {
+        out = device_tensor(base::DataType::DataTypeBf16, dims, device, file.data(*e), e->byte_size());
+        return base::error::success();
+    }
+    if (e->dtype != "F16" && e->dtype != "F32") return bad_file(name + ": expected BF16, F16 or F32");
+    std::vector<uint16_t> rounded(count);
+    if (e->dtype == "F32") {
+        const float* src = static_cast<const float*>(file.data(*e));
+        for (size_t i = 0; i < count; i++) rounded[i] = kernel::float_to_bf16(src[i]);
+    } else {
+        const uint16_t* src = static_cast<const uint16_t*>(file.data(*e));
+        for (size_t i = 0; i < count; i++) rounded[i] = kernel::float_to_bf16(kernel::fp16_to_float(src[i]));
+    }
+    out = device_tensor(base::DataType::DataTypeBf16, dims, device, rounded.data(), count * sizeof(uint16_t));
+    return base::error::success();
 }
 
 }  // namespace model

@@ -9,25 +9,6 @@
 namespace kernel {
 namespace {
 
-inline float half_to_float(uint16_t h) {
-    const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
-    const uint32_t exponent = (h >> 10) & 0x1fu;
-    const uint32_t mantissa = h & 0x3ffu;
-    uint32_t u;
-    if (exponent == 0) {
-        const float v = static_cast<float>(mantissa) * (1.0f / 16777216.0f);  // mantissa * 2^-24
-        std::memcpy(&u, &v, sizeof(u));
-        u |= sign;
-    } else if (exponent == 31) {
-        u = sign | 0x7f800000u | (mantissa << 13);
-    } else {
-        u = sign | ((exponent + 112u) << 23) | (mantissa << 13);
-    }
-    float f;
-    std::memcpy(&f, &u, sizeof(f));
-    return f;
-}
-
 // column of nibble i inside a packed word: 0, 2, 4, 6, 1, 3, 5, 7
 inline int column_of_nibble(int i) {
     return i < 4 ? 2 * i : 2 * (i - 4) + 1;
@@ -122,7 +103,7 @@ void matmul_kernel_awq_cpu(const tensor::Tensor& input, const tensor::Tensor& qw
                 for (int i = 0; i < 8; i++) {
                     const int32_t n = 8 * j + column_of_nibble(i);
                     const float z = static_cast<float>((zword >> (4 * i)) & 0xfu);
-                    total[n] += half_to_float(sc[static_cast<size_t>(g) * N + n]) * (qx[n] - z * xsum);
+                    total[n] += fp16_to_float(sc[static_cast<size_t>(g) * N + n]) * (qx[n] - z * xsum);
                 }
             }
         }
