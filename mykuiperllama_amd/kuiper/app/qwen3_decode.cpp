@@ -1,10 +1,14 @@
 // kx_qwen3_decode [--graph] [--max-positions N] file.safetensors token [token ...]
+// kx_qwen3_decode [--graph] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]
 //
-// Feeds the tokens one by one to model::Qwen3Decoder from an empty KV cache (token i at position i)
-// and prints one line per step:
+// First form: feeds the tokens one by one to model::Qwen3Decoder from an empty KV cache (token i at
+// position i) and prints one line per step:
 //     position token next_token fnv1a64-of-the-bf16-logits
-// With --graph the step is captured in a HIP graph first and every token replays it.  The model's
-// sizes are read off the checkpoint's tensors.
+// The model's sizes are read off the checkpoint's tensors.
+// Second form: random-init weights of the named architecture, caches filled with N(0,1) up to the
+// context length, then S steps at position C timed back to back; prints one JSON line with
+// ms_per_step and tokens_per_s (batch 1, lm_head and argmax included).
+// With --graph the step is captured in a HIP graph first and every step replays it.
 #include <cinttypes>
 #include <cstdio>
 #include <cstdlib>
@@ -14,24 +18,75 @@
 
 #include "model/qwen3_decoder.h"
 
+namespace {
+
+int run_random(const std::string& name, int32_t context, int32_t steps, int32_t warmup, bool graph) {
+    model::Qwen3Config c;
+    if (name == "qwen3-8b") {
+        c.layers = 36, c.hidden = 4096, c.intermediate = 12288, c.n_q_heads = 32, c.n_kv_heads = 8, c.vocab = 151936;
+    } else if (name == "qwen3-32b") {
+        c.layers = 64, c.hidden = 5120, c.intermediate = 25600, c.n_q_heads = 64, c.n_kv_heads = 8, c.vocab = 151936;
+    } else if (name == "tiny") {
+        c.layers = 2, c.hidden = 512, c.intermediate = 1024, c.n_q_heads = 4, c.n_kv_heads = 2, c.vocab = 1024;
+    } else {
+        std::fprintf(stderr, "unknown architecture %s (qwen3-8b, qwen3-32b, tiny)\n", name.c_str());
+        return 2;
+    }
+    if (context < 0 || steps < 1 || warmup < 0) {
+        std::fprintf(stderr, "--context C (>= 0), --steps S (>= 1) and --warmup W (>= 0) are needed with --random\n");
+        return 2;
+    }
+    model::Qwen3Decoder decoder(c, context + 1);
+    decoder.init_random(20251125);
+    decoder.fill_cache_random(context, 7);
+    base::Status st = graph ? decoder.capture() : base::error::success();
+    double ms = 0.0;
+    if (st) st = decoder.time_steps(17 % c.vocab, context, steps, warmup, &ms);
+    if (!st) {
+        std::fprintf(stderr, "%s\n", st.get_err_msg().c_str());
+        return 1;
+    }
+    std::printf("{\"model\": \"%s\", \"weights\": \"random-init\", \"context\": %d, \"graph\": %s, "
+                "\"launches_per_step\": %d, \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
+                "\"tokens_per_s\": %.2f}\n",
+                name.c_str(), context, graph ? "true" : "false", decoder.launches_per_step(), steps, warmup, ms,
+                1000.0 / ms);
+    return 0;
+}
+
+}  // namespace
+
 int main(int argc, char** argv) {
     bool graph = false;
-    int32_t max_positions = 0;
-    std::string path;
+    int32_t max_positions = 0, context = -1, steps = 50, warmup = 10;
+    std::string path, random_model;
     std::vector<int32_t> tokens;
+    auto number = [&](int& i) { return static_cast<int32_t>(std::strtol(argv[++i], nullptr, 10)); };
     for (int i = 1; i < argc; i++) {
         if (std::strcmp(argv[i], "--graph") == 0) {
             graph = true;
         } else if (std::strcmp(argv[i], "--max-positions") == 0 && i + 1 < argc) {
-            max_positions = static_cast<int32_t>(std::strtol(argv[++i], nullptr, 10));
+            max_positions = number(i);
+        } else if (std::strcmp(argv[i], "--context") == 0 && i + 1 < argc) {
+            context = number(i);
+        } else if (std::strcmp(argv[i], "--steps") == 0 && i + 1 < argc) {
+            steps = number(i);
+        } else if (std::strcmp(argv[i], "--warmup") == 0 && i + 1 < argc) {
+            warmup = number(i);
+        } else if (std::strcmp(argv[i], "--random") == 0 && i + 1 < argc) {
+            random_model = argv[++i];
         } else if (path.empty()) {
             path = argv[i];
         } else {
             tokens.push_back(static_cast<int32_t>(std::strtol(argv[i], nullptr, 10)));
         }
     }
+    if (!random_model.empty()) return run_random(random_model, context, steps, warmup, graph);
     if (path.empty() || tokens.empty()) {
-        std::fprintf(stderr, "usage: %s [--graph] [--max-positions N] file.safetensors token [token ...]\n", argv[0]);
+        std::fprintf(stderr,
+                     "usage: %s [--graph] [--max-positions N] file.safetensors token [token ...]\n"
+                     "       %s [--graph] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]\n",
+                     argv[0], argv[0]);
         return 2;
     }
     if (max_positions <= 0) max_positions = static_cast<int32_t>(tokens.size());

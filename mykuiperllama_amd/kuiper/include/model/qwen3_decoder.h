@@ -65,6 +65,13 @@ public:
     // unquantised tensors (F16 is rounded to bf16).
     base::Status load(const SafetensorsFile& file);
 
+    // Random-init weights of the configured architecture instead of a checkpoint (benchmarks): packed
+    // words uniform, scales sized so that activations keep O(1) magnitude through the layers, norm
+    // gains 1 + 0.02 N(0,1), embedding N(0,1), lm_head 0.02 N(0,1).  Seeded; nothing is read from disk.
+    void init_random(uint64_t seed);
+    // Rows 0 .. positions-1 of every cache set to bf16 N(0,1), the state a benchmark decodes from.
+    void fill_cache_random(int32_t positions, uint64_t seed);
+
     // One token at position pos (0 <= pos < max_positions): appends its key and value to the caches
     // and returns the most likely next token.  Synchronises the decoder's stream.
     base::Status step(int32_t token, int32_t pos, int32_t* next_token);
@@ -72,6 +79,10 @@ public:
     // Records the step in a HIP graph; later step() calls replay it.
     base::Status capture();
     bool captured() const { return graph_exec_ != nullptr; }
+
+    // `steps` steps of the same token at the same position back to back (after `warmup` untimed
+    // ones), timed with events on the decoder's stream; replays the graph when one is captured.
+    base::Status time_steps(int32_t token, int32_t pos, int32_t steps, int32_t warmup, double* ms_per_step);
 
     // bf16 logits of the last step, copied to the host.
     std::vector<uint16_t> logits() const;

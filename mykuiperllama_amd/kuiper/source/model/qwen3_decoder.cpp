@@ -4,10 +4,12 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 
 #include "base/alloc.h"
 #include "kx_hip.h"
+#include "random_fill.h"
 
 namespace model {
 namespace {
@@ -193,6 +195,94 @@ base::Status Qwen3Decoder::load(const SafetensorsFile& file) {
         if (!st) return st;
     }
     loaded_ = true;
+    return base::error::success();
+}
+
+void Qwen3Decoder::init_random(uint64_t seed) {
+    const Qwen3Config& c = config_;
+    void* s = stream();
+    uint64_t stream_id = 0;
+    auto next_seed = [&]() { return seed * 0x9E3779B97F4A7C15ull + (++stream_id << 40); };
+    auto random_awq = [&](op::MatmulLayer& layer) {
+        const int32_t N = layer.dim0(), K = layer.dim1(), G = layer.group_size();
+        tensor::Tensor qweight = device_tensor(base::DataType::DataTypeInt32, {K, N / 8});
+        tensor::Tensor qzeros = device_tensor(base::DataType::DataTypeInt32, {K / G, N / 8});
+        tensor::Tensor scales = device_tensor(base::DataType::DataTypeFp16, {K / G, N});
+        fill_random_words(qweight.ptr<int32_t>(), qweight.size(), next_seed(), s);
+        fill_random_words(qzeros.ptr<int32_t>(), qzeros.size(), next_seed(), s);
+        // |q - z| is about 4.6 on average: scales of 1 / (4.6 sqrt(K)) keep a row's magnitude
+        const float unit = 1.0f / (4.6f * std::sqrt(static_cast<float>(K)));
+        fill_uniform_fp16(scales.ptr<uint16_t>(), scales.size(), next_seed(), 0.75f * unit, 1.25f * unit, s);
+        CHECK(layer.set_weight(0, qweight));
+        CHECK(layer.set_weight(1, qzeros));
+        layer.set_awq_scales(scales);
+    };
+    auto random_bf16 = [&](const std::vector<int32_t>& dims, float mean, float std) {
+        tensor::Tensor t = device_tensor(base::DataType::DataTypeBf16, dims);
+        fill_normal_bf16(t.ptr<uint16_t>(), t.size(), next_seed(), mean, std, s);
+        return t;
+    };
+    for (LayerWeights& L : layers_) {
+        random_awq(*L.qkv);
+        random_awq(*L.o);
+        random_awq(*L.gate_up);
+        random_awq(*L.down);
+        L.input_norm = random_bf16({c.hidden}, 1.0f, 0.02f);
+        L.post_norm = random_bf16({c.hidden}, 1.0f, 0.02f);
+        L.q_norm = random_bf16({c.head_dim}, 1.0f, 0.02f);
+        L.k_norm = random_bf16({c.head_dim}, 1.0f, 0.02f);
+    }
+    embed_ = random_bf16({c.vocab, c.hidden}, 0.0f, 1.0f);
+    final_norm_ = random_bf16({c.hidden}, 1.0f, 0.02f);
+    CHECK(lm_head_->set_weight(0, random_bf16({c.vocab, c.hidden}, 0.0f, 0.02f)));
+    CHECK_EQ(hipStreamSynchronize(stream()), hipSuccess);
+    loaded_ = true;
+}
+
+void Qwen3Decoder::fill_cache_random(int32_t positions, uint64_t seed) {
+    CHECK_GE(positions, 0);
+    CHECK_LE(positions, max_positions_);
+    const size_t n = static_cast<size_t>(positions) * config_.n_kv_heads * config_.head_dim;
+    uint64_t id = 0;
+    for (LayerWeights& L : layers_) {
+        fill_normal_bf16(u16(L.k_cache), n, seed * 0xD1342543DE82EF95ull + (++id << 40), 0.0f, 1.0f, stream());
+        fill_normal_bf16(u16(L.v_cache), n, seed * 0xD1342543DE82EF95ull + (++id << 40), 0.0f, 1.0f, stream());
+    }
+    CHECK_EQ(hipStreamSynchronize(stream()), hipSuccess);
+}
+
+base::Status Qwen3Decoder::time_steps(int32_t token, int32_t pos, int32_t steps, int32_t warmup, double* ms_per_step) {
+    if (!loaded_) return base::error::invalid_argument("qwen3: no weights");
+    if (ms_per_step == nullptr || steps < 1 || warmup < 0) return base::error::invalid_argument("qwen3: bad arguments");
+    int32_t next = 0;
+    base::Status st = step(token, pos, &next);  // uploads token and position, checks them
+    if (!st) return st;
+    hipEvent_t begin = nullptr, end = nullptr;
+    if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
+        return base::error::internal_error("qwen3: event creation failed");
+    }
+    int rc = KX_OK;
+    hipError_t err = hipSuccess;
+    for (int32_t i = 0; i < warmup + steps && rc == KX_OK && err == hipSuccess; i++) {
+        if (i == warmup) err = hipEventRecord(begin, stream());
+        if (err != hipSuccess) break;
+        if (graph_exec_) {
+            err = hipGraphLaunch(graph_exec_, stream());
+        } else {
+            rc = enqueue_step();
+        }
+    }
+    if (rc == KX_OK && err == hipSuccess) err = hipEventRecord(end, stream());
+    const hipError_t sync = hipStreamSynchronize(stream());  // also after a failure: nothing may be left in flight
+    float ms = 0.0f;
+    if (rc == KX_OK && err == hipSuccess && sync == hipSuccess) err = hipEventElapsedTime(&ms, begin, end);
+    (void)hipEventDestroy(begin);
+    (void)hipEventDestroy(end);
+    if (rc != KX_OK) return base::error::internal_error(std::string("qwen3: launch failed: ") + kx_error_string(rc));
+    if (err != hipSuccess || sync != hipSuccess) {
+        return base::error::internal_error(std::string("qwen3: timing: ") + hipGetErrorString(err != hipSuccess ? err : sync));
+    }
+    *ms_per_step = static_cast<double>(ms) / steps;
     return base::error::success();
 }
 

@@ -107,3 +107,24 @@ def test_tool_reports_a_missing_file_and_a_file_without_a_model(tmp_path):
     assert "model.embed_tokens.weight" in done.stderr
     done = run_tool([])
     assert done.returncode == 2 and "usage" in done.stderr
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [[], ["--graph"]])
+def test_tool_times_a_random_init_model(mode):
+    import json
+    done = run_tool(mode + ["--random", "tiny", "--context", 300, "--steps", 20, "--warmup", 5])
+    assert done.returncode == 0, done.stderr
+    line = json.loads(done.stdout)
+    assert line["model"] == "tiny" and line["context"] == 300 and line["steps"] == 20
+    assert line["graph"] is bool(mode)
+    assert line["launches_per_step"] == 1 + 2 * 5 + 3
+    assert 0.0 < line["ms_per_step"] < 50.0
+    assert abs(line["tokens_per_s"] * line["ms_per_step"] - 1000.0) < 1.0
+
+
+def test_tool_rejects_an_unknown_architecture_and_a_missing_context():
+    done = run_tool(["--random", "qwen9-1t", "--context", 10])
+    assert done.returncode == 2 and "unknown architecture" in done.stderr
+    done = run_tool(["--random", "tiny"])
+    assert done.returncode == 2 and "--context" in done.stderr
