@@ -1,10 +1,11 @@
-// kx_qwen3_decode [--graph] [--max-positions N] file.safetensors token [token ...]
+// kx_qwen3_decode [--graph] [--max-positions N] [--generate N] file.safetensors token [token ...]
 // kx_qwen3_decode [--graph] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]
 //
 // First form: feeds the tokens one by one to model::Qwen3Decoder from an empty KV cache (token i at
 // position i) and prints one line per step:
 //     position token next_token fnv1a64-of-the-bf16-logits
-// The model's sizes are read off the checkpoint's tensors.
+// The model's sizes are read off the checkpoint's tensors.  With --generate N the greedy token is fed
+// back N more times after the last given token (lines continue in the same format).
 // Second form: random-init weights of the named architecture, caches filled with N(0,1) up to the
 // context length, then S steps at position C timed back to back; prints one JSON line with
 // ms_per_step and tokens_per_s (batch 1, lm_head and argmax included).
@@ -58,7 +59,7 @@ int run_random(const std::string& name, int32_t context, int32_t steps, int32_t 
 
 int main(int argc, char** argv) {
     bool graph = false;
-    int32_t max_positions = 0, context = -1, steps = 50, warmup = 10;
+    int32_t max_positions = 0, context = -1, steps = 50, warmup = 10, generate = 0;
     std::string path, random_model;
     std::vector<int32_t> tokens;
     auto number = [&](int& i) { return static_cast<int32_t>(std::strtol(argv[++i], nullptr, 10)); };
@@ -67,6 +68,8 @@ int main(int argc, char** argv) {
             graph = true;
         } else if (std::strcmp(argv[i], "--max-positions") == 0 && i + 1 < argc) {
             max_positions = number(i);
+        } else if (std::strcmp(argv[i], "--generate") == 0 && i + 1 < argc) {
+            generate = number(i);
         } else if (std::strcmp(argv[i], "--context") == 0 && i + 1 < argc) {
             context = number(i);
         } else if (std::strcmp(argv[i], "--steps") == 0 && i + 1 < argc) {
@@ -84,12 +87,18 @@ int main(int argc, char** argv) {
     if (!random_model.empty()) return run_random(random_model, context, steps, warmup, graph);
     if (path.empty() || tokens.empty()) {
         std::fprintf(stderr,
-                     "usage: %s [--graph] [--max-positions N] file.safetensors token [token ...]\n"
+                     "usage: %s [--graph] [--max-positions N] [--generate N] file.safetensors token [token ...]\n"
                      "       %s [--graph] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]\n",
                      argv[0], argv[0]);
         return 2;
     }
-    if (max_positions <= 0) max_positions = static_cast<int32_t>(tokens.size());
+    if (generate < 0) generate = 0;
+    const size_t total = tokens.size() + static_cast<size_t>(generate);
+    if (max_positions <= 0) max_positions = static_cast<int32_t>(total);
+    if (static_cast<size_t>(max_positions) < total) {
+        std::fprintf(stderr, "--max-positions %d is less than the %zu positions asked for\n", max_positions, total);
+        return 2;
+    }
 
     model::SafetensorsFile file;
     base::Status st = file.open(path);
@@ -111,7 +120,7 @@ int main(int argc, char** argv) {
     }
     file.close();  // the weights are on the GPU
     std::fprintf(stderr, "%d launches per step%s\n", decoder.launches_per_step(), graph ? ", one graph" : "");
-    for (size_t i = 0; i < tokens.size(); i++) {
+    for (size_t i = 0; i < total; i++) {
         int32_t next = -1;
         st = decoder.step(tokens[i], static_cast<int32_t>(i), &next);
         if (!st) {
@@ -126,6 +135,7 @@ int main(int argc, char** argv) {
             h *= 1099511628211ull;
         }
         std::printf("%zu %d %d %016" PRIx64 "\n", i, tokens[i], next, h);
+        if (i + 1 == tokens.size() && tokens.size() < total) tokens.push_back(next);  // greedy continuation
     }
     return 0;
 }

@@ -128,3 +128,29 @@ def test_tool_rejects_an_unknown_architecture_and_a_missing_context():
     assert done.returncode == 2 and "unknown architecture" in done.stderr
     done = run_tool(["--random", "tiny"])
     assert done.returncode == 2 and "--context" in done.stderr
+
+
+@pytest.mark.gpu
+def test_greedy_continuation_follows_the_python_driver(tmp_path, oracle):
+    import torch
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    layers_np, _, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
+    path = tmp_path / "model.safetensors"
+    write_checkpoint(path, torch, layers_np, embed, lm_head, final_norm)
+    prompt, more = [17, 3, 900], 9
+    model = decode.DecodeModel(cfg, len(prompt) + more, weights=to_model_weights(torch, layers_np, embed, lm_head, final_norm))
+    fed, expected = list(prompt), []
+    for pos in range(len(prompt) + more):
+        model.set_input(fed[pos], pos)
+        model.step(fused=True)
+        torch.cuda.synchronize()
+        nxt = int(model.next_token.item())
+        expected.append((pos, fed[pos], nxt, fnv1a64(model.logits.view(torch.int16).cpu().numpy().tobytes())))
+        if pos + 1 == len(fed):
+            fed.append(nxt)
+    done = run_tool(["--graph", "--generate", more, path] + prompt)
+    assert done.returncode == 0, done.stderr
+    assert parse(done.stdout) == expected
+    done = run_tool(["--max-positions", 5, "--generate", more, path] + prompt)
+    assert done.returncode == 2 and "--max-positions" in done.stderr
