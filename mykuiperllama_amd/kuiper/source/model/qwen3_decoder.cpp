@@ -34,7 +34,6 @@ std::unique_ptr<op::MatmulLayer> awq_layer(int32_t n, int32_t k, int32_t group) 
     return std::make_unique<op::MatmulLayer>(base::DeviceType::DeviceCUDA, n, k, true, group);
 }
 
-const uint16_t* u16(const tensor::Tensor& t) { return t.ptr<uint16_t>(); }
 uint16_t* u16(tensor::Tensor& t) { return t.ptr<uint16_t>(); }
 
 struct Awq {
