@@ -26,7 +26,12 @@
 #include "base/base.h"
 #include "base/cuda_config.h"
 #include "model/safetensors.h"
+#include "op/embedding.h"
 #include "op/matmul.h"
+#include "op/mha.h"
+#include "op/rmsnorm.h"
+#include "op/rope.h"
+#include "op/swiglu.h"
 #include "tensor/tensor.h"
 
 namespace model {
@@ -51,11 +56,19 @@ struct Qwen3Config {
     static base::Status from_file(const SafetensorsFile& file, Qwen3Config& config);
 };
 
+// How a step is put together.
+//   Fused   the fused entry points of kx_hip.h, five or six launches per decoder layer (the fast path)
+//   Layers  one kuiper layer per operator, forward() by forward() — EmbeddingLayer, RmsNormLayer (with
+//           the residual add in front), MatmulLayer, RoPELayer, MultiHeadAttention, SwiGLULayer — ten
+//           launches per decoder layer: what a model written against the layer API of
+//           kuiper/include/op/layer.h looks like, and the yardstick the fused path is held against
+enum class DecodePath { Fused, Layers };
+
 class Qwen3Decoder {
 public:
     // Allocates caches and scratch rows for max_positions positions.  The decoder runs on a stream
     // of its own (graph capture needs one that is not the default stream).
-    Qwen3Decoder(const Qwen3Config& config, int32_t max_positions);
+    Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, DecodePath path = DecodePath::Fused);
     ~Qwen3Decoder();
     Qwen3Decoder(const Qwen3Decoder&) = delete;
     Qwen3Decoder& operator=(const Qwen3Decoder&) = delete;
@@ -88,6 +101,7 @@ public:
     std::vector<uint16_t> logits() const;
 
     const Qwen3Config& config() const { return config_; }
+    DecodePath path() const { return path_; }
     int32_t max_positions() const { return max_positions_; }
     int32_t launches_per_step() const;
     hipStream_t stream() const { return stream_->stream(); }
@@ -99,10 +113,19 @@ private:
         tensor::Tensor k_cache, v_cache;
     };
 
+    struct LayerOps {
+        std::unique_ptr<op::RmsNormLayer> input_norm, post_norm;
+        std::unique_ptr<op::RoPELayer> rope;
+    };
+
     int enqueue_step();  // 0 or the first failing entry point's return code
+    int enqueue_step_fused();
+    int enqueue_step_layers();
+    void attach_layer_weights();  // Layers path: gains and tables into the operator layers
 
     Qwen3Config config_;
     int32_t max_positions_ = 0;
+    DecodePath path_ = DecodePath::Fused;
     bool merge_in_o_ = false;
     bool loaded_ = false;
     std::shared_ptr<kernel::CudaConfig> stream_;
@@ -110,6 +133,14 @@ private:
     tensor::Tensor embed_, final_norm_;
     std::unique_ptr<op::MatmulLayer> lm_head_;
     tensor::Tensor x_, h_, q_, attn_, gate_up_, logits_, sumsq_;
+    // Layers path only
+    std::vector<LayerOps> layer_ops_;
+    std::unique_ptr<op::EmbeddingLayer> embedding_op_;
+    std::unique_ptr<op::MultiHeadAttention> attention_op_;
+    std::unique_ptr<op::SwiGLULayer> swiglu_op_;
+    std::unique_ptr<op::RmsNormLayer> final_norm_op_;
+    tensor::Tensor qkv_, o_, act_, down_;
+    tensor::Tensor token_view_, pos_view_, gate_view_, up_view_;  // borrowed pieces of io_ and gate_up_
     tensor::Tensor gemv_workspace_, attn_workspace_;
     tensor::Tensor io_;           // device: token, position, next token (int32 each)
     int32_t* host_io_ = nullptr;  // pinned mirror of io_

@@ -20,6 +20,9 @@ public:
     base::Status check() const override;
     base::Status forward() override;
     using TypedLayer::forward;
+    // Allocates the GPU workspace for caches of max_positions rows now, so that forward() allocates
+    // nothing later (a stream under graph capture must not).  No effect on a host layer.
+    base::Status reserve(int32_t max_positions);
 
 private:
     int32_t n_q_ = 0;

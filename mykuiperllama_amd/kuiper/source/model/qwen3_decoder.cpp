@@ -8,6 +8,7 @@
 #include <cstdlib>
 
 #include "base/alloc.h"
+#include "kernel/hip/matmul_kernel.h"
 #include "kx_hip.h"
 #include "random_fill.h"
 
@@ -91,8 +92,8 @@ base::Status Qwen3Config::from_file(const SafetensorsFile& file, Qwen3Config& co
     return base::error::success();
 }
 
-Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions)
-    : config_(config), max_positions_(max_positions) {
+Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, DecodePath path)
+    : config_(config), max_positions_(max_positions), path_(path) {
     const Qwen3Config& c = config_;
     CHECK_EQ(c.head_dim, 128) << "the attention and rotary kernels are built for heads of 128";
     CHECK_GT(c.layers, 0);
@@ -147,6 +148,49 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions)
     attn_workspace_ = device_bytes(attn_bytes);
 
     CHECK_EQ(hipHostMalloc(reinterpret_cast<void**>(&host_io_), 3 * sizeof(int32_t), hipHostMallocDefault), hipSuccess);
+
+    if (path_ == DecodePath::Layers) {
+        const base::DeviceType gpu = base::DeviceType::DeviceCUDA;
+        qkv_ = device_tensor(bf16, {c.qkv_out()});
+        o_ = device_tensor(bf16, {c.hidden});
+        act_ = device_tensor(bf16, {c.intermediate});
+        down_ = device_tensor(bf16, {c.hidden});
+        auto borrowed = [&](base::DataType type, int32_t n, void* ptr) {
+            tensor::Tensor t(type, n, false, nullptr, ptr);
+            t.set_device_type(gpu);  // a borrowed buffer does not know where it lives
+            return t;
+        };
+        token_view_ = borrowed(base::DataType::DataTypeInt32, 1, io_.ptr<int32_t>());
+        pos_view_ = borrowed(base::DataType::DataTypeInt32, 1, io_.ptr<int32_t>() + 1);
+        gate_view_ = borrowed(bf16, c.intermediate, u16(gate_up_));
+        up_view_ = borrowed(bf16, c.intermediate, u16(gate_up_) + c.intermediate);
+        embedding_op_ = std::make_unique<op::EmbeddingLayer>(gpu, c.vocab, c.hidden);
+        attention_op_ = std::make_unique<op::MultiHeadAttention>(gpu, c.n_q_heads, c.n_kv_heads);
+        swiglu_op_ = std::make_unique<op::SwiGLULayer>(gpu, c.intermediate);
+        final_norm_op_ = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
+        embedding_op_->set_cuda_config(stream_);
+        attention_op_->set_cuda_config(stream_);
+        swiglu_op_->set_cuda_config(stream_);
+        final_norm_op_->set_cuda_config(stream_);
+        lm_head_->set_cuda_config(stream_);
+        layer_ops_.resize(layers_.size());
+        for (size_t i = 0; i < layers_.size(); i++) {
+            LayerOps& ops = layer_ops_[i];
+            ops.input_norm = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
+            ops.post_norm = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
+            ops.rope = std::make_unique<op::RoPELayer>(gpu, c.n_q_heads, c.n_kv_heads, c.rope_theta, c.rms_eps);
+            ops.input_norm->set_cuda_config(stream_);
+            ops.post_norm->set_cuda_config(stream_);
+            ops.rope->set_cuda_config(stream_);
+            layers_[i].qkv->set_cuda_config(stream_);
+            layers_[i].o->set_cuda_config(stream_);
+            layers_[i].gate_up->set_cuda_config(stream_);
+            layers_[i].down->set_cuda_config(stream_);
+        }
+        // everything a forward() would allocate on first use, now: a captured stream must not allocate
+        CHECK(attention_op_->reserve(max_positions));
+        kernel::matmul_reserve_workspace(stream(), 1, big_k, big_n);
+    }
     CHECK_EQ(hipStreamSynchronize(stream()), hipSuccess);
 }
 
@@ -194,7 +238,20 @@ base::Status Qwen3Decoder::load(const SafetensorsFile& file) {
         if (!st) return st;
     }
     loaded_ = true;
+    attach_layer_weights();
     return base::error::success();
+}
+
+void Qwen3Decoder::attach_layer_weights() {
+    if (path_ != DecodePath::Layers) return;
+    CHECK(embedding_op_->set_weight(0, embed_));
+    CHECK(final_norm_op_->set_weight(0, final_norm_));
+    for (size_t i = 0; i < layers_.size(); i++) {
+        CHECK(layer_ops_[i].input_norm->set_weight(0, layers_[i].input_norm));
+        CHECK(layer_ops_[i].post_norm->set_weight(0, layers_[i].post_norm));
+        CHECK(layer_ops_[i].rope->set_weight(0, layers_[i].q_norm));
+        CHECK(layer_ops_[i].rope->set_weight(1, layers_[i].k_norm));
+    }
 }
 
 void Qwen3Decoder::init_random(uint64_t seed) {
@@ -236,6 +293,7 @@ void Qwen3Decoder::init_random(uint64_t seed) {
     CHECK(lm_head_->set_weight(0, random_bf16({c.vocab, c.hidden}, 0.0f, 0.02f)));
     CHECK_EQ(hipStreamSynchronize(stream()), hipSuccess);
     loaded_ = true;
+    attach_layer_weights();
 }
 
 void Qwen3Decoder::fill_cache_random(int32_t positions, uint64_t seed) {
@@ -286,10 +344,52 @@ base::Status Qwen3Decoder::time_steps(int32_t token, int32_t pos, int32_t steps,
 }
 
 int32_t Qwen3Decoder::launches_per_step() const {
-    return 1 + config_.layers * (merge_in_o_ ? 5 : 6) + 3;  // embedding; layers; final norm, lm_head, argmax
+    const int32_t per_layer = path_ == DecodePath::Layers ? 10 : (merge_in_o_ ? 5 : 6);
+    return 1 + config_.layers * per_layer + 3;  // embedding; layers; final norm, lm_head, argmax
 }
 
 int Qwen3Decoder::enqueue_step() {
+    return path_ == DecodePath::Layers ? enqueue_step_layers() : enqueue_step_fused();
+}
+
+// One forward() per operator, in the order of the model's formulas.  A layer reports a refused
+// tensor through its Status; a failed launch aborts inside the layer's kernel wrapper, as in the
+// reference's GPU wrappers.
+int Qwen3Decoder::enqueue_step_layers() {
+    const Qwen3Config& c = config_;
+#define KX_LAYER(call)                          \
+    do {                                        \
+        const base::Status layer_status = call; \
+        if (!layer_status) {                    \
+            LOG(ERROR) << layer_status.get_err_msg(); \
+            return KX_ERR_BAD_SHAPE;            \
+        }                                       \
+    } while (0)
+    KX_LAYER(embedding_op_->forward(token_view_, x_));
+    for (int32_t li = 0; li < c.layers; li++) {
+        LayerWeights& L = layers_[static_cast<size_t>(li)];
+        LayerOps& ops = layer_ops_[static_cast<size_t>(li)];
+        if (li == 0) {
+            KX_LAYER(ops.input_norm->forward(x_, h_));
+        } else {
+            KX_LAYER(ops.input_norm->forward(x_, down_, h_));  // x += down of the previous layer, then the norm
+        }
+        KX_LAYER(L.qkv->forward(h_, qkv_));
+        KX_LAYER(ops.rope->forward(qkv_, pos_view_, L.k_cache, L.v_cache, q_));
+        KX_LAYER(attention_op_->forward(q_, pos_view_, L.k_cache, L.v_cache, attn_));
+        KX_LAYER(L.o->forward(attn_, o_));
+        KX_LAYER(ops.post_norm->forward(x_, o_, h_));
+        KX_LAYER(L.gate_up->forward(h_, gate_up_));
+        KX_LAYER(swiglu_op_->forward(gate_view_, up_view_, act_));
+        KX_LAYER(L.down->forward(act_, down_));
+    }
+    KX_LAYER(final_norm_op_->forward(x_, down_, h_));
+    KX_LAYER(lm_head_->forward(h_, logits_));
+#undef KX_LAYER
+    return kx_argmax_bf16(u16(logits_), c.vocab, io_.ptr<int32_t>() + 2, stream());
+}
+
+int Qwen3Decoder::enqueue_step_fused() {
     const Qwen3Config& c = config_;
     void* s = stream();
     void* ws = gemv_workspace_.ptr<uint8_t>();

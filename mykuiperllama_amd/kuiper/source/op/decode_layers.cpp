@@ -235,6 +235,17 @@ base::Status MultiHeadAttention::forward() {
     return base::error::success();
 }
 
+base::Status MultiHeadAttention::reserve(int32_t max_positions) {
+    if (device_type_ != base::DeviceType::DeviceCUDA) return base::error::success();
+    const size_t need = kx_attn_decode_workspace_bytes(n_q_, kHeadDim, max_positions);
+    if (need == 0) return base::error::invalid_argument("mha: no attention kernel for this head layout or context length");
+    if (workspace_.is_empty() || workspace_.byte_size() < need) {
+        workspace_ = tensor::Tensor(base::DataType::DataTypeInt8, static_cast<int32_t>(need), true,
+                                    base::CUDADeviceAllocatorFactory::get_instance());
+    }
+    return base::error::success();
+}
+
 #undef KX_RETURN_IF_BAD
 
 }  // namespace op

@@ -19,6 +19,10 @@ void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qwe
 // Releases every cached workspace (for orderly shutdown in tests).
 void matmul_release_workspaces();
 
+// Makes the workspace of `stream` large enough for a GEMV of this shape now, so that later launches
+// on that stream allocate nothing (a stream under graph capture must not).
+void matmul_reserve_workspace(void* stream, int32_t M, int32_t K, int32_t N);
+
 }  // namespace kernel
 
 #endif  // KUIPER_KERNEL_HIP_MATMUL_KERNEL_H

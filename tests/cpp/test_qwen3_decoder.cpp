@@ -202,3 +202,44 @@ TEST_GPU(test_qwen3_decoder, random_init_depends_on_the_seed_only) {
     ASSERT_TRUE(bool(a.time_steps(100, 1, 3, 1, &ms)));
     ASSERT_TRUE(ms > 0.0);
 }
+
+TEST_GPU(test_qwen3_decoder, layer_by_layer_path_agrees_with_the_fused_path) {
+    // Same weights, same tokens: one forward() per operator against the fused entry points.  The fused
+    // path adds up the sum of squares of the RMSNorm tile by tile, so the logits agree to rounding.
+    model::Qwen3Decoder fused(tiny_config(), 64), layers(tiny_config(), 64, model::DecodePath::Layers);
+    fused.init_random(11);
+    layers.init_random(11);
+    ASSERT_TRUE(layers.path() == model::DecodePath::Layers);
+    ASSERT_EQ(layers.launches_per_step(), 1 + 2 * 10 + 3);
+    const int32_t tokens[] = {9, 400, 77, 1000, 3, 3};
+    for (int i = 0; i < 6; i++) {
+        int32_t a = -1, b = -1;
+        ASSERT_TRUE(bool(fused.step(tokens[i], i, &a)));
+        ASSERT_TRUE(bool(layers.step(tokens[i], i, &b)));
+        const std::vector<uint16_t> la = fused.logits(), lb = layers.logits();
+        double num = 0.0, den = 0.0;
+        for (size_t k = 0; k < la.size(); k++) {
+            const double x = kxo_bf16_to_f32(la[k]), y = kxo_bf16_to_f32(lb[k]);
+            num += (x - y) * (x - y);
+            den += y * y;
+        }
+        ASSERT_TRUE(den > 0.0);
+        ASSERT_LE(std::sqrt(num / den), 2e-2);
+    }
+}
+
+TEST_GPU(test_qwen3_decoder, layer_by_layer_path_can_be_captured) {
+    model::Qwen3Decoder eager(tiny_config(), 40, model::DecodePath::Layers);
+    model::Qwen3Decoder replayed(tiny_config(), 40, model::DecodePath::Layers);
+    eager.init_random(5);
+    replayed.init_random(5);
+    ASSERT_TRUE(bool(replayed.capture()));  // nothing may allocate while the stream is captured
+    for (int i = 0; i < 5; i++) {
+        int32_t a = -1, b = -2;
+        ASSERT_TRUE(bool(eager.step(100 + i, i, &a)));
+        ASSERT_TRUE(bool(replayed.step(100 + i, i, &b)));
+        ASSERT_EQ(a, b);
+        const std::vector<uint16_t> la = eager.logits(), lb = replayed.logits();
+        ASSERT_EQ(std::memcmp(la.data(), lb.data(), la.size() * 2), 0);
+    }
+}

@@ -65,6 +65,33 @@ def parse(stdout):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("max_positions", [48, 6000])
+def test_cpp_decoder_built_from_layers_matches_the_unfused_python_step(tmp_path, oracle, max_positions):
+    """--layers: one kuiper layer forward() per operator; DecodeModel.step(fused=False) enqueues the same
+    ten launches per decoder layer through the C ABI."""
+    import torch
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(**CFG)
+    layers_np, _, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
+    path = tmp_path / "model.safetensors"
+    write_checkpoint(path, torch, layers_np, embed, lm_head, final_norm)
+    model = decode.DecodeModel(cfg, max_positions, weights=to_model_weights(torch, layers_np, embed, lm_head, final_norm))
+    expected = []
+    for pos, token in enumerate(TOKENS):
+        model.set_input(token, pos)
+        model.step(fused=False)
+        torch.cuda.synchronize()
+        logits = model.logits.view(torch.int16).cpu().numpy().tobytes()
+        expected.append((pos, token, int(model.next_token.item()), fnv1a64(logits)))
+    for mode in (["--layers"], ["--layers", "--graph"]):
+        done = run_tool(mode + ["--max-positions", max_positions, path] + TOKENS)
+        assert done.returncode == 0, done.stderr
+        launches = model.launches_per_step(with_lm_head=True, fused=False)
+        assert f"{launches} launches per step" in done.stderr
+        assert parse(done.stdout) == expected, (mode, done.stderr)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("max_positions,tied", [(48, False), (6000, False), (10368, False), (48, True)])
 def test_cpp_decoder_matches_the_python_driver_bit_for_bit(tmp_path, oracle, max_positions, tied):
     import torch
