@@ -196,6 +196,7 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
 
 Qwen3Decoder::~Qwen3Decoder() {
     if (stream_) (void)hipStreamSynchronize(stream());
+    if (stream_ && path_ == DecodePath::Layers) kernel::matmul_release_workspace(stream());  // the stream goes away with us
     if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_) (void)hipGraphDestroy(graph_);
     if (host_io_) (void)hipHostFree(host_io_);

@@ -57,6 +57,10 @@ void matmul_release_workspaces() {
     workspaces().clear();
 }
 
+void matmul_release_workspace(void* stream) {
+    workspaces().erase(stream);
+}
+
 void matmul_reserve_workspace(void* stream, int32_t M, int32_t K, int32_t N) {
     (void)workspace_for(stream, kx_gemv_workspace_bytes(M, K, N));
 }

@@ -18,6 +18,9 @@ void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qwe
 
 // Releases every cached workspace (for orderly shutdown in tests).
 void matmul_release_workspaces();
+// Releases the workspace of one stream; whoever destroys a stream calls this first, so that a later
+// stream that happens to get the same handle starts without an entry.
+void matmul_release_workspace(void* stream);
 
 // Makes the workspace of `stream` large enough for a GEMV of this shape now, so that later launches
 // on that stream allocate nothing (a stream under graph capture must not).
