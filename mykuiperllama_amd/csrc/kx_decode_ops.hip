@@ -331,6 +331,23 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
     const int kvh = head / G;
     const int g = head % G;
     const int tid = threadIdx.x;
+    // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...
+    const int d = tid % kHeadDim;
+    const int part = tid / kHeadDim;
+    const float* po = part_out + (static_cast<size_t>(kvh) * nchunks * G + g) * kHeadDim + d;
+    const size_t cstride = static_cast<size_t>(G) * kHeadDim;
+    // The partial sums do not depend on the rescaling factors: the first kMergeFront chunks of this
+    // thread are requested before the statistics, so the kernel costs one trip to memory for both
+    // instead of one for the statistics and one per batch of eight chunks after it.  Clamped
+    // addresses, masked use: straight-line loads.
+    constexpr int kMergeFront = 32;  // chunks per thread in that first flight: 128 chunks of the context
+    float front[kMergeFront];
+#pragma unroll
+    for (int u = 0; u < kMergeFront; u++) {
+        const int c = part + u * kMergeParts;
+        front[u] = po[(c < nchunks ? c : nchunks - 1) * cstride];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (tid < kWave) {
         const MergeStats<kMergeLanesLong> st =
             attn_merge_load<kMergeLanesLong>(part_ml + static_cast<size_t>(kvh) * nchunks * G * 2, g, G, nchunks, tid);
@@ -339,13 +356,14 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
     }
     __syncthreads();
 
-    // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...
-    const int d = tid % kHeadDim;
-    const int part = tid / kHeadDim;
-    const float* po = part_out + (static_cast<size_t>(kvh) * nchunks * G + g) * kHeadDim + d;
-    const size_t cstride = static_cast<size_t>(G) * kHeadDim;
     float acc = 0.0f;
-    for (int c0 = part; c0 < nchunks; c0 += kMergeBatch * kMergeParts) {
+#pragma unroll
+    for (int u = 0; u < kMergeFront; u++) {
+        const int c = part + u * kMergeParts;
+        if (c < nchunks) acc = attn_merge_step(acc, front[u], s_factor[c]);
+    }
+    // what a longer context leaves, in batches as before; the order of the additions is unchanged
+    for (int c0 = part + kMergeFront * kMergeParts; c0 < nchunks; c0 += kMergeBatch * kMergeParts) {
         float v[kMergeBatch];
 #pragma unroll
         for (int u = 0; u < kMergeBatch; u++) {
