@@ -444,11 +444,32 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* 
     const int chunks = wide ? n / 8 : 0;
     const uint4* xv = reinterpret_cast<const uint4*>(x);
 
+    // First sweep: twenty 16-byte loads per thread, all in flight together and kept in registers —
+    // the 151 936 logits of the Qwen3 vocabulary are one sweep, i.e. one trip to memory, and the
+    // search for the index below needs no second one.  Clamped addresses: straight-line loads; a
+    // piece past the end re-reads the last one, which cannot change a maximum.
     float mine = -INFINITY;  // fmaxf drops a NaN operand
-    constexpr int kInFlight = 8;  // 16-byte loads per thread and sweep
-    for (int c0 = tid; c0 < chunks; c0 += kInFlight * kArgmaxThreads) {
-        // clamped addresses: the loads of a sweep are straight-line code, all in flight together;
-        // a piece past the end re-reads the last one, which cannot change a maximum
+    constexpr int kHeld = 20;
+    uint4 held[kHeld];
+#pragma unroll
+    for (int u = 0; u < kHeld; u++) held[u] = make_uint4(0u, 0u, 0u, 0u);
+    if (chunks > 0) {  // nothing is read from an input without a whole 16-byte piece
+#pragma unroll
+        for (int u = 0; u < kHeld; u++) {
+            const int c = tid + u * kArgmaxThreads;
+            held[u] = xv[c < chunks ? c : chunks - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < kHeld; u++) {
+            float v[8];
+            unpack8(held[u], v);
+#pragma unroll
+            for (int i = 0; i < 8; i++) mine = fmaxf(mine, v[i]);
+        }
+    }
+    // longer inputs: further sweeps of eight loads
+    constexpr int kInFlight = 8;
+    for (int c0 = tid + kHeld * kArgmaxThreads; c0 < chunks; c0 += kInFlight * kArgmaxThreads) {
         uint4 raw[kInFlight];
 #pragma unroll
         for (int u = 0; u < kInFlight; u++) {
@@ -473,16 +494,28 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* 
 
     int first = 0x7fffffff;
     if (mine == best) {  // few threads: they walk their own elements again (-0 and +0 are one value)
-        for (int c = tid; c < chunks; c += kArgmaxThreads) {
+#pragma unroll
+        for (int u = kHeld - 1; u >= 0; u--) {  // the held pieces, from registers
+            const int c = tid + u * kArgmaxThreads;
             float v[8];
-            unpack8(xv[c], v);
+            unpack8(held[u], v);
 #pragma unroll
             for (int i = 7; i >= 0; i--) {
-                if (v[i] == best && 8 * c + i < first) first = 8 * c + i;
+                if (c < chunks && v[i] == best) first = 8 * c + i;  // descending walk: the last hit is the first index
             }
         }
-        for (int i = 8 * chunks + tid; i < n; i += kArgmaxThreads) {
-            if (bf16_to_f32(x[i]) == best && i < first) first = i;
+        if (first == 0x7fffffff) {  // not among the held pieces: the later sweeps, re-read
+            for (int c = tid + kHeld * kArgmaxThreads; c < chunks; c += kArgmaxThreads) {
+                float v[8];
+                unpack8(xv[c], v);
+#pragma unroll
+                for (int i = 7; i >= 0; i--) {
+                    if (v[i] == best && 8 * c + i < first) first = 8 * c + i;
+                }
+            }
+            for (int i = 8 * chunks + tid; i < n; i += kArgmaxThreads) {
+                if (bf16_to_f32(x[i]) == best && i < first) first = i;
+            }
         }
     }
 #pragma unroll
