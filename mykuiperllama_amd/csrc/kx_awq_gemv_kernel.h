@@ -178,6 +178,16 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         const int col = ct * kTileCols + tid % kTileCols;
         resid_pre = res.in[col < N ? col : N - 1];
     }
+    int rope_pos = 0;
+    uint16_t rope_gain_a = 0, rope_gain_b = 0;
+    if constexpr (EPI == kEpiQkRope) {
+        // what the wave that finishes head 2 ct + (tid / 128) will need, see the epilogue below
+        const int head = ct * (kTileCols / kHeadDim) + ((tid % kTileCols) >> 7);
+        const uint16_t* gain = head < rope.n_q ? rope.q_gain : rope.k_gain;
+        rope_gain_a = gain[tid % kWave];
+        rope_gain_b = gain[tid % kWave + 64];
+        rope_pos = rope.pos[0];
+    }
     float tile_ss = 0.0f;
     if constexpr (PRO == kProPreNorm) {
         const int part = tid % kWave;
@@ -520,7 +530,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         if (tid < kTileCols && (tid & 64) == 0) {
             const int local = tid >> 7;
             const int head = ct * (kTileCols / kHeadDim) + local;
-            qk_norm_rope_head(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane, rope);
+            qk_norm_rope_head_with(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane, rope,
+                                   rope_pos, rope_gain_a, rope_gain_b);
         }
     }
 }

@@ -31,9 +31,12 @@ struct RopeTarget {
 //   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
 //   out[i + 64] = x[i+64] * cos(pos f_i) + x[i] * sin(pos f_i),     f_i = theta^(-i/64)
 // where x is the head after RMSNorm (rounded to bf16, as a bf16 norm layer returns it).
-__device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bits, int head, int lane,
-                                                  const RopeTarget& t) {
-    const int pos = t.pos[0];
+// `pos`, `gain_a` and `gain_b` are *t.pos and elements lane and lane + 64 of the head's gain (q_gain for a
+// query head, k_gain for a key head, unused for a value head): a caller that knows early which head
+// a wave will serve loads them ahead of time.
+__device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t b_bits, int head, int lane,
+                                                       const RopeTarget& t, int pos, uint16_t gain_a,
+                                                       uint16_t gain_b) {
     const bool row_ok = static_cast<unsigned>(pos) < static_cast<unsigned>(t.cache_positions);
     if (head >= t.n_q + t.n_kv) {  // value head: straight into the cache
         if (row_ok) {
@@ -46,11 +49,10 @@ __device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bi
     const float a = bf16_to_f32(a_bits);
     const float b = bf16_to_f32(b_bits);
     const bool is_q = head < t.n_q;
-    const uint16_t* gain = is_q ? t.q_gain : t.k_gain;
     const float ss = wave_sum(a * a + b * b);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(kHeadDim) + t.eps);
-    const float na = bf16_to_f32(gain[lane]) * bf16_to_f32(f32_to_bf16(a * inv));
-    const float nb = bf16_to_f32(gain[lane + 64]) * bf16_to_f32(f32_to_bf16(b * inv));
+    const float na = bf16_to_f32(gain_a) * bf16_to_f32(f32_to_bf16(a * inv));
+    const float nb = bf16_to_f32(gain_b) * bf16_to_f32(f32_to_bf16(b * inv));
     // the norm output is a bf16 tensor in the usual formulation; the rotation starts from that
     const float xa = bf16_to_f32(f32_to_bf16(na));
     const float xb = bf16_to_f32(f32_to_bf16(nb));
@@ -65,6 +67,13 @@ __device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bi
         dst[lane] = f32_to_bf16(oa);
         dst[lane + 64] = f32_to_bf16(ob);
     }
+}
+
+// The same with the three operands loaded here.
+__device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bits, int head, int lane,
+                                                  const RopeTarget& t) {
+    const uint16_t* gain = head < t.n_q ? t.q_gain : t.k_gain;  // a value head reads k_gain and ignores it
+    qk_norm_rope_head_with(a_bits, b_bits, head, lane, t, t.pos[0], gain[lane], gain[lane + 64]);
 }
 
 }  // namespace kx
