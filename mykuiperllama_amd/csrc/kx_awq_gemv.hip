@@ -73,7 +73,10 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
     // 9.1 / 9.3 / -: the minimum of that cost picks the faster one every time.
     // (Twelve waves of 32 rows, 768 rows per workgroup and one workgroup per compute unit on down
     // 12288->4096, are faster still on the plain launch, 9.0 -> 8.6 us, but slower with the SwiGLU
-    // prologue of the decode step, whose latency then has no second workgroup to hide behind.)
+    // prologue of the decode step, whose latency then has no second workgroup to hide behind.  Eight
+    // waves of eight rows, 128 rows per workgroup, for projections too narrow to give every compute
+    // unit a workgroup — k 4096->1024 has 64 — are slower as well, 5.07 -> 5.48 us: twice the K tiles
+    // to exchange cost more than the idle compute units.)
     // Twelve waves: one activation row, plain or SwiGLU input, plain or residual output only (the
     // other prologues and epilogues are laid out for 4 or 8 waves).  Shorter K than 256 takes fewer
     // waves so that no workgroup is mostly idle.
