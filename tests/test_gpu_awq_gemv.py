@@ -80,7 +80,7 @@ def test_gemv_m1_matches_oracle(capi, torch, oracle, K, N):
 
 
 @pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 16])
-@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 1024), (12288, 4096)])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 1024), (12288, 4096), (4096, 12288), (4096, 24576)])
 def test_gemv_small_batch_matches_oracle(capi, torch, oracle, M, K, N):
     p = synth.make_awq_problem(f"gemv_m{M}_{K}x{N}", M, K, N)
     y, _ = run_awq(capi, torch, p)

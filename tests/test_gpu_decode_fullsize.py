@@ -1,0 +1,135 @@
+"""Decode-step parity at the full benchmark configurations: the whole Qwen3-8B step (36 layers, hidden 4096,
+context 4096) and the Qwen3-32B-shaped step (64 layers, hidden 5120, context 8192), random-init weights.
+
+These sizes select launch plans the small model of test_gpu_decode_step.py never reaches together (12-wave
+and 32-rows-per-lane workgroups, the long add+norm prologue, the attention merge inside and outside the o
+projection, 128-position attention chunks).  The reference has no model code to compare with
+(its CMakeLists.txt:79 names a model directory that is absent), so the pins are: the ten-launch step built
+from the stand-alone operators (each of which has its own oracle / torch test), bit for bit; a HIP-graph
+replay, bit for bit; and one decoder layer at full width against the fp32 restatement fed with the CPU
+oracle's dequantised weights.
+"""
+import pytest
+
+from tests.test_gpu_decode_step import Reference, make_weights, to_model_weights
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch as _t
+    assert _t.cuda.is_available()
+    return _t
+
+
+def _bits(t, torch):
+    return t.view(torch.int16)
+
+
+def _run_tokens(model, torch, mode, tokens, ctx):
+    """Feed `tokens` at positions ctx, ctx+1, ...; returns per-step (logits, residual stream, next token)."""
+    out = []
+    for i, tok in enumerate(tokens):
+        model.set_input(tok, ctx + i)
+        model.step(fused=mode)
+        torch.cuda.synchronize()
+        out.append((model.logits.clone(), int(model.next_token.item())))
+    return out
+
+
+@pytest.mark.parametrize("name,ctx", [("qwen3-8b", 4096), ("qwen3-32b", 8192)])
+def test_full_size_step_fused_unfused_chained_and_graph(torch, name, ctx):
+    from mykuiperllama_amd import decode
+    cfg = {"qwen3-8b": decode.QWEN3_8B, "qwen3-32b": decode.QWEN3_32B}[name]
+    print(f"full-size decode parity: {name} layers={cfg.layers} hidden={cfg.hidden} ctx={ctx}", flush=True)
+    model = decode.DecodeModel(cfg, max_positions=ctx + 128)
+    model.prefill_cache_random(ctx)
+
+    # three consecutive tokens, greedy, on the ten-launch path; the other paths are fed the same tokens
+    tokens = [11]
+    base = []
+    for i in range(3):
+        model.set_input(tokens[-1], ctx + i)
+        model.step(fused=False)
+        torch.cuda.synchronize()
+        base.append((model.logits.clone(), int(model.next_token.item())))
+        tokens.append(base[-1][1])
+    tokens = tokens[:3]
+    for logits, _ in base:
+        assert torch.isfinite(logits.float()).all()
+
+    # (i) the small operators inside the GEMV launches: bit for bit the ten-launch step
+    fused = _run_tokens(model, torch, "prologue", tokens, ctx)
+    for i, ((la, ta), (lb, tb)) in enumerate(zip(base, fused)):
+        assert torch.equal(_bits(la, torch), _bits(lb, torch)), f"{name}: prologue step differs at token {i}"
+        assert ta == tb
+
+    # (ii) chained launches: the RMSNorm's sum of squares is added tile by tile, equal up to that rounding
+    chained = _run_tokens(model, torch, "chain", tokens, ctx)
+    for i, ((la, _), (lb, _)) in enumerate(zip(base, chained)):
+        la, lb = la.float(), lb.float()
+        assert torch.isfinite(lb).all()
+        err = ((la - lb).norm() / la.norm()).item()
+        assert err <= 5e-3, f"{name}: chained step off by {err} at token {i}"
+
+    # (iii) a captured step replayed bitwise equals the same step launched eagerly
+    for mode in ("chain", "prologue"):
+        model.set_input(tokens[2], ctx + 2)
+        model.step(fused=mode)
+        torch.cuda.synchronize()
+        eager = model.logits.clone()
+        eager_tok = int(model.next_token.item())
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                model.step(fused=mode)
+            for _ in range(2):
+                model.logits.zero_()
+                torch.cuda.synchronize()
+                g.replay()
+                side.synchronize()
+                assert torch.equal(_bits(model.logits, torch), _bits(eager, torch)), f"{name}: graph replay ({mode})"
+                assert int(model.next_token.item()) == eager_tok
+        torch.cuda.synchronize()
+        del g
+    del model
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("hidden,inter,n_q,n_kv,ctx", [(4096, 12288, 32, 8, 4096), (5120, 25600, 64, 8, 8192)])
+def test_one_full_width_layer_matches_the_fp32_reference(torch, oracle, hidden, inter, n_q, n_kv, ctx):
+    """One decoder layer at the real widths and context against the torch fp32 restatement with separate
+    projections whose weights are the CPU oracle's dequantisation (relative L2 <= 2e-2, as for the small
+    model), on each of the three launch paths."""
+    from mykuiperllama_amd import decode
+    cfg = decode.ModelConfig(layers=1, hidden=hidden, intermediate=inter, n_q=n_q, n_kv=n_kv, vocab=1024)
+    layers_np, layers_ref, embed, lm_head, final_norm = make_weights(torch, oracle, cfg)
+    weights = to_model_weights(torch, layers_np, embed, lm_head, final_norm)
+    del layers_np
+    for mode in (True, "prologue", False):
+        print(f"full-width layer: hidden={hidden} intermediate={inter} heads={n_q}/{n_kv} ctx={ctx} mode={mode}",
+              flush=True)
+        model = decode.DecodeModel(cfg, ctx + 128, weights=weights)
+        model.prefill_cache_random(ctx)
+        ref = Reference(torch, cfg, layers_ref, embed, lm_head, final_norm,
+                        [k.cpu() for k in model.k_cache], [v.cpu() for v in model.v_cache])
+        token = 17
+        for stepno in range(2):
+            pos = ctx + stepno
+            model.set_input(token, pos)
+            model.step(fused=mode)
+            torch.cuda.synchronize()
+            x_ref, logits_ref = ref.step(token, pos)
+            got = model.logits[0].cpu().float()
+            assert torch.isfinite(got).all()
+            err = ((got - logits_ref.float()).norm() / logits_ref.float().norm()).item()
+            assert err <= 2e-2, f"mode {mode} step {stepno}: logits relative L2 {err}"
+            xerr = ((model.x[0].cpu().float() - x_ref.float()).norm() / x_ref.float().norm()).item()
+            assert xerr <= 2e-2, f"mode {mode} step {stepno}: residual stream relative L2 {xerr}"
+            kerr = (model.k_cache[0][pos].cpu().float() - ref.k[0][pos].float()).abs().max().item()
+            assert kerr <= 0.06
+            token = int(logits_ref.float().argmax())
+        del model, ref
+        torch.cuda.empty_cache()
