@@ -80,13 +80,9 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
                      const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
                      int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Two kernels implement kx_gemv_awq_bf16: one on the vector ALUs (used for M = 1) and one on the
- * matrix cores (MFMA; used for M >= 2 when the group size is a power of two and N a multiple of
- * sixteen).  This knob overrides the choice for tuning and for tests: 0 = by shape (default),
- * 1 = always the vector kernel, 2 = the MFMA kernel wherever group size and N allow.
- * Process-wide, not thread-safe.
- * Reference counterpart: none. */
-int kx_set_awq_kernel_policy(int policy);
+/* Two kernels implement kx_gemv_awq_bf16, chosen by shape: one on the vector ALUs and one on the matrix
+ * cores (MFMA; M >= 2, and wide projections at M = 1, when the group size is a power of two and N a
+ * multiple of sixteen).  The library keeps no state about the choice. */
 
 /* ------------------------------------------------------------------------------------------
  * The same GEMV with the activations produced on the way in, for the decode step (one launch

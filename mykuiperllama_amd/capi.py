@@ -21,7 +21,6 @@ SIGNATURES = {
     "kx_gemv_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kx_workspace_init": (ctypes.c_int, [_P, _SZ, _P]),
     "kx_gemv_awq_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
-    "kx_set_awq_kernel_policy": (ctypes.c_int, [ctypes.c_int]),
     "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_swiglu_bf16": (ctypes.c_int, [_P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_addnorm_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I32, _I32,
@@ -45,6 +44,12 @@ SIGNATURES = {
     "kx_embedding_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _P]),
     "kx_argmax_bf16": (ctypes.c_int, [_P, _I32, _P, _P]),
     "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
+}
+
+
+# entry points outside the drop-in boundary (csrc/kx_internal.h): tests and the benchmark only
+INTERNAL_SIGNATURES = {
+    "kx_gemv_awq_bf16_policy": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P, _I32]),
 }
 
 
@@ -91,7 +96,7 @@ def load():
             f"{KX_LIB} is missing: the HIP library has not been built "
             "(python -m mykuiperllama_amd.build). There is no CPU fallback for this path.")
     lib = ctypes.CDLL(KX_LIB)
-    for name, (res, args) in SIGNATURES.items():
+    for name, (res, args) in list(SIGNATURES.items()) + list(INTERNAL_SIGNATURES.items()):
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
@@ -130,6 +135,11 @@ def gemv_awq_bf16(x, qweight, scales, qzeros, y, group_size, workspace):
     """x bf16 [M,K], qweight int32 [K,N/8], scales fp16 [K/G,N], qzeros int32 [K/G,N/8], y bf16 [M,N]."""
     M, K = x.shape
     N = y.shape[-1]
+    if _policy != 0:
+        _check(load().kx_gemv_awq_bf16_policy(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
+                                              M, K, N, group_size, _ptr(workspace),
+                                              0 if workspace is None else workspace.numel(), _stream(), _policy))
+        return
     _check(load().kx_gemv_awq_bf16(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
                                    M, K, N, group_size, _ptr(workspace),
                                    0 if workspace is None else workspace.numel(), _stream()))
@@ -171,9 +181,18 @@ def gemv_awq_qkv_rope_bf16(residual, delta, gain, eps, residual_out, qweight, sc
                                             0 if workspace is None else workspace.numel(), _stream()))
 
 
+_policy = 0
+
+
 def set_awq_kernel_policy(policy):
-    """0 = choose by shape, 1 = vector-ALU kernel, 2 = MFMA kernel where group size and N allow."""
-    _check(load().kx_set_awq_kernel_policy(policy))
+    """Test and benchmark plumbing: which kernel gemv_awq_bf16 of THIS module asks for from now on.
+    0 = the product entry point (the library chooses by shape); 1 = vector-ALU kernel, 2 = one-shot MFMA
+    kernel, each through the internal entry point kx_gemv_awq_bf16_policy.
+    The library itself keeps no such state."""
+    global _policy
+    if policy not in (0, 1, 2):
+        raise ValueError("policy must be 0, 1 or 2")
+    _policy = policy
 
 
 def gemv_bf16(x, w, y, workspace=None):

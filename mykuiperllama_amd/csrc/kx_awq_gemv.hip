@@ -1,6 +1,7 @@
 // Host side of the fused INT4 AWQ dequantise + GEMV: shape checks, launch plan, C ABI.
 #include "kx_awq_gemv_kernel.h"
 #include "kx_awq_gemv_mfma_kernel.h"
+#include "kx_internal.h"
 
 
 namespace kx {
@@ -18,13 +19,6 @@ struct AwqPlan {
 
 inline int rows_per_block(int waves, int rt) {
     return waves * kSlotsPerWave * rt;
-}
-
-// 0: choose by shape; 1: always the VALU kernel; 2: the MFMA kernel wherever group size and N allow
-int g_kernel_policy = 0;
-
-inline int kernel_override() {
-    return g_kernel_policy;
 }
 
 constexpr int kComputeUnits = 256;  // MI355X
@@ -108,12 +102,17 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
     return p;
 }
 
-inline AwqPlan make_plan(int M, int K, int N, int group) {
+inline AwqPlan make_plan(int M, int K, int N, int group, int mode) {
     // The MFMA kernel needs quantisation groups that tile the workgroup's K range (powers of two)
     // and loads two packed words at a time (N a multiple of sixteen).
     const bool mfma_ok = is_pow2(group) && (N % 16) == 0;
-    const int mode = kernel_override();
-    const bool mfma = mfma_ok && (mode == 2 || (mode == 0 && M >= 2));
+    // One activation row: the two kernels are within a few per cent of each other; the MFMA kernel is the
+    // faster one on wide projections of moderate K (us per launch, vector / MFMA: 4096->12288 8.9 / 8.5,
+    // 4096->24576 13.5 / 13.0, 5120->10240 11.0 / 10.5, 5120->51200 30.9 / 29.3), the vector kernel on
+    // narrow ones and on tall K, where its 384- and 512-row workgroups exchange fewer partial sums
+    // (4096->4096 5.7 / 5.8, 12288->4096 9.2 / 9.6, 25600->5120 18.6 / 19.5).
+    const bool wide_m1 = M == 1 && N >= 8192 && K <= 8192;
+    const bool mfma = mfma_ok && (mode == KX_POLICY_MFMA || (mode == KX_POLICY_BY_SHAPE && (M >= 2 || wide_m1)));
     return mfma ? make_mfma_plan(M, K, N, group) : make_valu_plan(M, K, N);
 }
 
@@ -216,18 +215,12 @@ __global__ void fill_zero_u32(uint32_t* p, size_t n) {
 }  // namespace
 }  // namespace kx
 
-extern "C" int kx_set_awq_kernel_policy(int policy) {
-    if (policy < 0 || policy > 2) return KX_ERR_BAD_SHAPE;
-    kx::g_kernel_policy = policy;
-    return KX_OK;
-}
-
 extern "C" size_t kx_gemv_workspace_bytes(int32_t M, int32_t K, int32_t N) {
     if (M < 1 || M > KX_MAX_BATCH || K < 1 || N < 8) return 0;
     // Either kernel may serve a shape (the group size and M decide); size for the larger exchange.
     const int kt_valu = kx::make_valu_plan(M, K, N, true, false).ktiles;  // the entry points that keep 8 waves exchange more
     const int kt_mfma = kx::make_mfma_plan(M, K, N, 32).ktiles;  // the smallest group gives the most K tiles
-    const size_t ktiles = static_cast<size_t>(kt_valu > kt_mfma ? kt_valu : kt_mfma);
+    size_t ktiles = static_cast<size_t>(kt_valu > kt_mfma ? kt_valu : kt_mfma);
     return kx::kCounterBytes + ktiles * M * static_cast<size_t>(N) * sizeof(float);
 }
 
@@ -246,11 +239,20 @@ extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const
                                 const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
                                 int32_t group_size, void* workspace, size_t workspace_bytes,
                                 void* stream) {
+    return kx_gemv_awq_bf16_policy(x, qweight, scales, qzeros, y, M, K, N, group_size, workspace, workspace_bytes,
+                                   stream, KX_POLICY_BY_SHAPE);
+}
+
+extern "C" int kx_gemv_awq_bf16_policy(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
+                                       const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
+                                       int32_t group_size, void* workspace, size_t workspace_bytes,
+                                       void* stream, int32_t policy) {
+    if (policy < KX_POLICY_BY_SHAPE || policy > KX_POLICY_MFMA) return KX_ERR_BAD_SHAPE;
     if (!x) return KX_ERR_NULL_POINTER;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
     if (rc != KX_OK) return rc;
     if (reinterpret_cast<uintptr_t>(x) % 16) return KX_ERR_ALIGNMENT;
-    kx::AwqPlan p = kx::make_plan(M, K, N, group_size);
+    kx::AwqPlan p = kx::make_plan(M, K, N, group_size, policy);
     float* partials = nullptr;
     uint32_t* counters = nullptr;
     rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
