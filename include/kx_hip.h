@@ -81,8 +81,7 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
                      int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Two kernels implement kx_gemv_awq_bf16, chosen by shape: one on the vector ALUs and one on the matrix
- * cores (MFMA; M >= 2, and wide projections at M = 1, when the group size is a power of two and N a
- * multiple of sixteen).  The library keeps no state about the choice. */
+ * cores (MFMA; M >= 2 when the group size is a power of two and N a multiple of sixteen).  The library keeps no state about the choice. */
 
 /* ------------------------------------------------------------------------------------------
  * The same GEMV with the activations produced on the way in, for the decode step (one launch

@@ -106,13 +106,12 @@ inline AwqPlan make_plan(int M, int K, int N, int group, int mode) {
     // The MFMA kernel needs quantisation groups that tile the workgroup's K range (powers of two)
     // and loads two packed words at a time (N a multiple of sixteen).
     const bool mfma_ok = is_pow2(group) && (N % 16) == 0;
-    // One activation row: the two kernels are within a few per cent of each other; the MFMA kernel is the
-    // faster one on wide projections of moderate K (us per launch, vector / MFMA: 4096->12288 8.9 / 8.5,
-    // 4096->24576 13.5 / 13.0, 5120->10240 11.0 / 10.5, 5120->51200 30.9 / 29.3), the vector kernel on
-    // narrow ones and on tall K, where its 384- and 512-row workgroups exchange fewer partial sums
-    // (4096->4096 5.7 / 5.8, 12288->4096 9.2 / 9.6, 25600->5120 18.6 / 19.5).
-    const bool wide_m1 = M == 1 && N >= 8192 && K <= 8192;
-    const bool mfma = mfma_ok && (mode == KX_POLICY_MFMA || (mode == KX_POLICY_BY_SHAPE && (M >= 2 || wide_m1)));
+    // One activation row stays on the vector kernel although the MFMA kernel is a few per cent faster on
+    // wide projections (us per launch, vector / MFMA: 4096->12288 8.9 / 8.5, 4096->24576 13.5 / 13.0,
+    // 5120->51200 30.9 / 29.3; narrow and tall ones the other way round: 4096->4096 5.7 / 5.8, 12288->4096
+    // 9.2 / 9.6): the launches with an activation prologue run on the vector kernel, and a plain launch
+    // returns their bits only if it adds in the same order.
+    const bool mfma = mfma_ok && (mode == KX_POLICY_MFMA || (mode == KX_POLICY_BY_SHAPE && M >= 2));
     return mfma ? make_mfma_plan(M, K, N, group) : make_valu_plan(M, K, N);
 }
 

@@ -27,6 +27,8 @@ public:
 private:
     int32_t n_q_ = 0;
     int32_t n_kv_ = 0;
+    base::Status grow_workspace(size_t need);
+
     tensor::Tensor workspace_;  // GPU only
 };
 

@@ -1,10 +1,14 @@
 // Stream ownership (reference: kuiper/source/base/cuda_config.cpp:4-23).
 #include "base/cuda_config.h"
 
+#include "kernel/hip/matmul_kernel.h"
+
 namespace kernel {
 
 CudaConfig::~CudaConfig() {
     if (stream_ != nullptr) {
+        // what the matmul wrapper keeps for this stream goes with it: a later stream may get the same handle
+        matmul_release_workspace(stream_);
         hipError_t err = hipStreamDestroy(stream_);
         if (err != hipSuccess) {
             // a destructor must not throw through a test's fatal handler: report only
@@ -20,6 +24,9 @@ void CudaConfig::create() {
 }
 
 hipStream_t CudaConfig::stream() const { return stream_; }
-void CudaConfig::set_stream(hipStream_t stream) { stream_ = stream; }
+void CudaConfig::set_stream(hipStream_t stream) {
+    if (stream_ != nullptr && stream_ != stream) matmul_release_workspace(stream_);
+    stream_ = stream;
+}
 
 }  // namespace kernel

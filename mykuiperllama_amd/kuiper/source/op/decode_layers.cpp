@@ -3,6 +3,8 @@
 // the layer's stream.
 #include <string>
 
+#include <hip/hip_runtime_api.h>
+
 #include "kernel/kernel_interface.h"
 #include "kx_hip.h"
 #include "op/embedding.h"
@@ -220,15 +222,34 @@ base::Status MultiHeadAttention::check() const {
     return base::error::success();
 }
 
+// Makes the attention workspace at least `need` bytes.  The block it replaces may still be read and
+// written by launches already enqueued on the layer's stream, and the allocator's pool would hand it
+// out again at once, so the stream is drained first; while the stream records a graph neither that wait
+// nor the allocation is possible, and the caller has to have reserved beforehand.
+base::Status MultiHeadAttention::grow_workspace(size_t need) {
+    if (!workspace_.is_empty() && workspace_.byte_size() >= need) return base::error::success();
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream()), &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusNone;
+    }
+    if (capture != hipStreamCaptureStatusNone) {
+        return base::error::invalid_argument(
+            "mha: the attention workspace must grow while the stream is capturing; call reserve(max_positions) "
+            "before the capture begins");
+    }
+    if (!workspace_.is_empty()) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream()));
+    workspace_ = tensor::Tensor(base::DataType::DataTypeInt8, static_cast<int32_t>(need), true,
+                                base::CUDADeviceAllocatorFactory::get_instance());
+    return base::error::success();
+}
+
 base::Status MultiHeadAttention::forward() {
     const base::Status status = check();
     if (!status) return status;
     if (device_type_ == base::DeviceType::DeviceCUDA) {
-        const size_t need = kx_attn_decode_workspace_bytes(n_q_, kHeadDim, get_input(2).get_dim(0));
-        if (workspace_.is_empty() || workspace_.byte_size() < need) {
-            workspace_ = tensor::Tensor(base::DataType::DataTypeInt8, static_cast<int32_t>(need), true,
-                                        base::CUDADeviceAllocatorFactory::get_instance());
-        }
+        const base::Status grown = grow_workspace(kx_attn_decode_workspace_bytes(n_q_, kHeadDim, get_input(2).get_dim(0)));
+        if (!grown) return grown;
     }
     kernel::get_mha_kernel(device_type_)(get_input(0), get_input(2), get_input(3), get_input(1), workspace_,
                                          get_output(0), n_q_, n_kv_, stream());
@@ -239,11 +260,7 @@ base::Status MultiHeadAttention::reserve(int32_t max_positions) {
     if (device_type_ != base::DeviceType::DeviceCUDA) return base::error::success();
     const size_t need = kx_attn_decode_workspace_bytes(n_q_, kHeadDim, max_positions);
     if (need == 0) return base::error::invalid_argument("mha: no attention kernel for this head layout or context length");
-    if (workspace_.is_empty() || workspace_.byte_size() < need) {
-        workspace_ = tensor::Tensor(base::DataType::DataTypeInt8, static_cast<int32_t>(need), true,
-                                    base::CUDADeviceAllocatorFactory::get_instance());
-    }
-    return base::error::success();
+    return grow_workspace(need);
 }
 
 #undef KX_RETURN_IF_BAD

@@ -23,12 +23,27 @@ std::map<void*, Workspace>& workspaces() {
     return table;
 }
 
+bool stream_is_capturing(void* stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &status) != hipSuccess) {
+        (void)hipGetLastError();  // a stream that cannot be asked is treated as not capturing
+        return false;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
 void* workspace_for(void* stream, size_t bytes) {
     if (bytes == 0) {
         return nullptr;
     }
     Workspace& ws = workspaces()[stream];
     if (ws.buffer == nullptr || ws.buffer->byte_size() < bytes) {
+        // Growing means allocating, waiting for the stream and initialising counters: none of that may
+        // happen while the stream records a graph (it would be refused, or end up inside the graph).
+        CHECK(!stream_is_capturing(stream))
+            << "the matmul workspace of this stream must grow to " << bytes
+            << " bytes while the stream is capturing: call kernel::matmul_reserve_workspace(stream, M, K, N) "
+               "for the largest projection before the capture begins";
         if (ws.buffer != nullptr) {
             // the old buffer may still be in use by launches already enqueued on this stream
             (void)hipStreamSynchronize(static_cast<hipStream_t>(stream));

@@ -8,6 +8,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../../mykuiperllama_amd/kuiper/source/op/kernel/hip/matmul_kernel.h"
 #include "../../mykuiperllama_amd/kuiper/source/op/kernel/kernel_interface.h"
 #include "../../oracle/kx_oracle.h"
 #include "mini_test.h"
@@ -263,4 +264,51 @@ TEST_GPU(test_matmul, kernel_interface_direct_call_on_default_stream) {
     y.to_cpu();
     std::memcpy(out.data(), y.ptr<uint16_t>(), out.size() * 2);
     expect_close(out, oracle_awq(p));
+}
+
+TEST_GPU(test_matmul, capture_without_a_reserved_workspace_is_refused_and_with_one_it_replays) {
+    // A stream that records a graph must not be synchronised or handed fresh allocations: the wrapper
+    // refuses to grow the split-K workspace then, and says what to call beforehand.
+    AwqProblem p = make_problem(1, 2048, 512, 128, 2718);
+    op::MatmulLayer layer(base::DeviceType::DeviceCUDA, p.N, p.K, true, p.G);
+    tensor::Tensor qw = host_tensor(base::DataType::DataTypeInt32, {p.K, p.N / 8}, p.qweight);
+    tensor::Tensor qz = host_tensor(base::DataType::DataTypeInt32, {p.K / p.G, p.N / 8}, p.qzeros);
+    tensor::Tensor sc = host_tensor(base::DataType::DataTypeFp16, {p.K / p.G, p.N}, p.scales);
+    tensor::Tensor x = host_tensor(base::DataType::DataTypeBf16, {p.M, p.K}, p.x);
+    std::vector<uint16_t> out(size_t(p.M) * p.N, 0x7FC0);
+    tensor::Tensor y = host_tensor(base::DataType::DataTypeBf16, {p.M, p.N}, out);
+    for (tensor::Tensor* t : {&qw, &qz, &sc, &x, &y}) t->to_cuda();
+    auto config = std::make_shared<kernel::CudaConfig>();
+    config->create();
+    layer.set_cuda_config(config);
+    ASSERT_TRUE(bool(layer.set_weight(0, qw)));
+    ASSERT_TRUE(bool(layer.set_weight(1, qz)));
+    layer.set_awq_scales(sc);
+    hipStream_t stream = config->stream();
+
+    hipGraph_t graph = nullptr;
+    ASSERT_EQ(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), hipSuccess);
+    ASSERT_FATAL(layer.forward(x, y));  // this stream has no workspace yet
+    ASSERT_EQ(hipStreamEndCapture(stream, &graph), hipSuccess);  // the capture itself is intact, and empty
+    if (graph != nullptr) ASSERT_EQ(hipGraphDestroy(graph), hipSuccess);
+
+    kernel::matmul_reserve_workspace(stream, p.M, p.K, p.N);
+    graph = nullptr;
+    ASSERT_EQ(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), hipSuccess);
+    ASSERT_TRUE(bool(layer.forward(x, y)));
+    ASSERT_EQ(hipStreamEndCapture(stream, &graph), hipSuccess);
+    ASSERT_NE(graph, nullptr);
+    hipGraphExec_t exec = nullptr;
+    ASSERT_EQ(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), hipSuccess);
+    for (int replay = 0; replay < 2; replay++) {
+        ASSERT_EQ(hipMemsetAsync(y.ptr<void>(), 0xFF, y.byte_size(), stream), hipSuccess);  // outside the graph
+        ASSERT_EQ(hipGraphLaunch(exec, stream), hipSuccess);
+        ASSERT_EQ(hipStreamSynchronize(stream), hipSuccess);
+        tensor::Tensor back = y.clone();
+        back.to_cpu();
+        std::memcpy(out.data(), back.ptr<uint16_t>(), out.size() * 2);
+        expect_close(out, oracle_awq(p));
+    }
+    ASSERT_EQ(hipGraphExecDestroy(exec), hipSuccess);
+    ASSERT_EQ(hipGraphDestroy(graph), hipSuccess);
 }
