@@ -83,6 +83,23 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
 /* Two kernels implement kx_gemv_awq_bf16, chosen by shape: one on the vector ALUs and one on the matrix
  * cores (MFMA; M >= 2 when the group size is a power of two and N a multiple of sixteen).  The library keeps no state about the choice. */
 
+/* kx_gemv_awq_bf16 for callers that cannot allocate or hand over a workspace (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc): the split-K workspace is a static device array inside
+ * the library, kx_gemv_awq_static_scratch_bytes() bytes (64 KiB of counters + 8 MiB of partial sums) per GPU
+ * the library runs on, held until the process ends.  Same arguments, kernels and bits as kx_gemv_awq_bf16.
+ * A shape whose kx_gemv_workspace_bytes(M, K, N) exceeds the array is rejected with KX_ERR_WORKSPACE and
+ * nothing is launched (every Qwen3-8B and -32B projection fits at M = 1, the 8B ones up to M = 4).
+ * Calls no hipMalloc / hipFree.  The first call on a device looks the array's address up and enqueues
+ * one small kernel that zeroes the counters; make that call outside stream capture.  All calls on one GPU
+ * share that GPU's array: calls that may overlap (different streams) race - use kx_gemv_awq_bf16 with
+ * separate workspaces for those.
+ * Reference counterpart: none (the reference has no split reduction and allocates through
+ * base::CUDADeviceAllocator only, kuiper/source/base/alloc_cu.cpp:8-16); it exists for the callers named above. */
+size_t kx_gemv_awq_static_scratch_bytes(void);
+int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
+                            const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
+                            int32_t group_size, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * The same GEMV with the activations produced on the way in, for the decode step (one launch
  * instead of two; built for M = 1, correct for M <= KX_MAX_BATCH, always the vector kernel).

@@ -21,6 +21,8 @@ SIGNATURES = {
     "kx_gemv_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kx_workspace_init": (ctypes.c_int, [_P, _SZ, _P]),
     "kx_gemv_awq_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
+    "kx_gemv_awq_static_scratch_bytes": (_SZ, []),
+    "kx_gemv_awq_bf16_static": (ctypes.c_int, [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P]),
     "kx_gemv_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_swiglu_bf16": (ctypes.c_int, [_P, _P, _I32, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
     "kx_gemv_awq_addnorm_bf16": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I32, _I32,
@@ -143,6 +145,14 @@ def gemv_awq_bf16(x, qweight, scales, qzeros, y, group_size, workspace):
     _check(load().kx_gemv_awq_bf16(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
                                    M, K, N, group_size, _ptr(workspace),
                                    0 if workspace is None else workspace.numel(), _stream()))
+
+
+def gemv_awq_bf16_static(x, qweight, scales, qzeros, y, group_size):
+    """gemv_awq_bf16 on the library's static scratch array: no workspace, no allocation."""
+    M, K = x.shape
+    N = y.shape[-1]
+    _check(load().kx_gemv_awq_bf16_static(_ptr(x), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(y),
+                                          M, K, N, group_size, _stream()))
 
 
 def gemv_awq_swiglu_bf16(gate, up, qweight, scales, qzeros, y, group_size, workspace):

@@ -3,6 +3,8 @@
 #include "kx_awq_gemv_mfma_kernel.h"
 #include "kx_internal.h"
 
+#include <mutex>
+
 
 namespace kx {
 namespace {
@@ -232,6 +234,70 @@ extern "C" int kx_workspace_init(void* workspace, size_t workspace_bytes, void* 
     hipLaunchKernelGGL(kx::fill_zero_u32, dim3((n + 255) / 256), dim3(256), 0, kx::as_stream(stream),
                        static_cast<uint32_t*>(workspace), n);
     return kx::launch_status();
+}
+
+// ---- the entry point that allocates nothing ----
+// The split-K workspace of kx_gemv_awq_bf16_static: arrival counters, then partial sums.  Every GPU the
+// library runs on holds its own copy of this array until the process ends.
+namespace {
+
+constexpr size_t kStaticPartialBytes = static_cast<size_t>(8) << 20;
+constexpr size_t kStaticScratchBytes = kx::kCounterBytes + kStaticPartialBytes;
+constexpr int kMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+struct StaticScratch {
+    std::mutex mu;
+    void* ptr[kMaxDevices] = {};  // device address of `scratch` on each device, null until first use there
+};
+
+StaticScratch g_static_scratch;
+
+// Device address of the current device's copy of `scratch`; on the first call on a device the address is
+// looked up and the arrival counters are zeroed on `stream` (a kernel, so that a capturing stream records
+// it like any other launch).  In host code the array's name is not a device address: only the pointer
+// obtained here is ever handed to a kernel.
+int static_scratch_for_current_device(void** out, hipStream_t stream) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return KX_ERR_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(g_static_scratch.mu);
+    if (!g_static_scratch.ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!p || reinterpret_cast<uintptr_t>(p) % 256) return KX_ERR_ALIGNMENT;
+        const size_t n = kx::kCounterBytes / sizeof(uint32_t);
+        hipLaunchKernelGGL(kx::fill_zero_u32, dim3((n + 255) / 256), dim3(256), 0, stream, static_cast<uint32_t*>(p), n);
+        const int rc = kx::launch_status();
+        if (rc != KX_OK) return rc;
+        g_static_scratch.ptr[dev] = p;
+    }
+    *out = g_static_scratch.ptr[dev];
+    return KX_OK;
+}
+
+}  // namespace
+
+extern "C" size_t kx_gemv_awq_static_scratch_bytes(void) {
+    return kStaticScratchBytes;
+}
+
+extern "C" int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
+                                       const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
+                                       int32_t group_size, void* stream) {
+    // argument errors first, so that a rejected call touches nothing
+    if (!x) return KX_ERR_NULL_POINTER;
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
+    if (rc != KX_OK) return rc;
+    if (kx_gemv_workspace_bytes(M, K, N) > kStaticScratchBytes) return KX_ERR_WORKSPACE;  // larger than the static array
+    void* ws = nullptr;
+    rc = static_scratch_for_current_device(&ws, kx::as_stream(stream));
+    if (rc != KX_OK) return rc;
+    return kx_gemv_awq_bf16_policy(x, qweight, scales, qzeros, y, M, K, N, group_size, ws, kStaticScratchBytes, stream,
+                                   KX_POLICY_BY_SHAPE);
 }
 
 extern "C" int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
