@@ -4,6 +4,11 @@
   libkuiper.so   C++ host API over that C ABI    (kuiper/source/**/*.cpp)
   test_kuiper    C++ test runner for the host API (tests/cpp/*, links oracle/kx_oracle.c)
   kx_safetensors_dump   lists the tensors of a checkpoint file (kuiper/app/safetensors_dump.cpp)
+  libkx_probe.so  measurement only: the streaming-read kernel bench.py uses as the floor (probe/*.hip)
+
+`python -m mykuiperllama_amd.build --ablate N` additionally builds lib/libkx_hip_ablateN.so, the HIP
+library with parts of the GEMV kernels compiled out (-DKX_ABLATE=N: 1 = no split-K exchange, 2 = loads
+only); `bench.py --lib` times it.  Its results are wrong by construction: it exists to attribute time.
 
 Everything lands under mykuiperllama_amd/lib/, in-tree, so that a snapshot of the repository
 carries the binaries to a machine that only runs them.
@@ -25,6 +30,8 @@ KUIPER_LIB = os.path.join(LIB_DIR, "libkuiper.so")
 KUIPER_TEST = os.path.join(LIB_DIR, "test_kuiper")
 SAFETENSORS_DUMP = os.path.join(LIB_DIR, "kx_safetensors_dump")
 QWEN3_DECODE = os.path.join(LIB_DIR, "kx_qwen3_decode")
+PROBE_LIB = os.path.join(LIB_DIR, "libkx_probe.so")
+PROBE_SRC = os.path.join(PKG, "probe")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU forms are switched off for all device code
@@ -40,11 +47,20 @@ def _run(cmd):
     return out
 
 
-def build_kx():
+def build_kx(ablate=0):
     os.makedirs(LIB_DIR, exist_ok=True)
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
-    _run([HIPCC] + DEVICE_FLAGS + COMMON + ["-shared", "-I", INCLUDE, "-I", CSRC] + srcs + ["-o", KX_LIB])
-    return KX_LIB
+    out = KX_LIB if not ablate else os.path.join(LIB_DIR, f"libkx_hip_ablate{int(ablate)}.so")
+    defines = [f"-DKX_ABLATE={int(ablate)}"] if ablate else []
+    _run([HIPCC] + DEVICE_FLAGS + COMMON + defines + ["-shared", "-I", INCLUDE, "-I", CSRC] + srcs + ["-o", out])
+    return out
+
+
+def build_probe():
+    os.makedirs(LIB_DIR, exist_ok=True)
+    srcs = sorted(glob.glob(os.path.join(PROBE_SRC, "*.hip")))
+    _run([HIPCC] + DEVICE_FLAGS + COMMON + ["-shared"] + srcs + ["-o", PROBE_LIB])
+    return PROBE_LIB
 
 
 def build_kuiper():
@@ -80,8 +96,15 @@ def build_kuiper():
 def build_all():
     build_kx()
     build_kuiper()
+    build_probe()
 
 
 if __name__ == "__main__":
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--ablate", type=int, default=0, help="also build lib/libkx_hip_ablateN.so (profiling only)")
+    args = ap.parse_args()
     build_all()
-    print("built:", KX_LIB, KUIPER_LIB if os.path.exists(KUIPER_LIB) else "")
+    print("built:", KX_LIB, KUIPER_LIB if os.path.exists(KUIPER_LIB) else "", PROBE_LIB)
+    if args.ablate:
+        print("built:", build_kx(args.ablate))

@@ -85,25 +85,50 @@ class KxError(RuntimeError):
 _lib = None
 
 
-def load():
-    """Load libkx_hip.so; raises if it has not been built."""
+def load(path=None):
+    """Load libkx_hip.so; raises if it has not been built.  `path` names another build of the library (the
+    benchmark's --lib, for profiling builds); it only has an effect on the first call."""
     global _lib
     if _lib is not None:
         return _lib
+    lib_path = path or KX_LIB
     # torch ships its own HIP runtime; it has to be in the process first so that this library
     # binds to the same copy (two runtimes in one process do not share a device context).
     import torch  # noqa: F401
-    if not os.path.exists(KX_LIB):
+    if not os.path.exists(lib_path):
         raise RuntimeError(
-            f"{KX_LIB} is missing: the HIP library has not been built "
+            f"{lib_path} is missing: the HIP library has not been built "
             "(python -m mykuiperllama_amd.build). There is no CPU fallback for this path.")
-    lib = ctypes.CDLL(KX_LIB)
+    lib = ctypes.CDLL(lib_path)
     for name, (res, args) in list(SIGNATURES.items()) + list(INTERNAL_SIGNATURES.items()):
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+_probe = None
+
+
+def probe_stream_read(buffers, sink=None):
+    """Measurement only: read up to three device tensors once with plain 16-byte loads (libkx_probe.so)."""
+    global _probe
+    if _probe is None:
+        import torch  # noqa: F401
+        from .build import PROBE_LIB
+        if not os.path.exists(PROBE_LIB):
+            raise RuntimeError(f"{PROBE_LIB} is missing (python -m mykuiperllama_amd.build)")
+        _probe = ctypes.CDLL(PROBE_LIB)
+        _probe.kx_probe_stream_read.restype = ctypes.c_int
+        _probe.kx_probe_stream_read.argtypes = [_P, _SZ, _P, _SZ, _P, _SZ, _P, _P]
+    args = []
+    for i in range(3):
+        t = buffers[i] if i < len(buffers) else None
+        args += [_ptr(t), 0 if t is None else t.numel() * t.element_size()]
+    rc = _probe.kx_probe_stream_read(*args, _ptr(sink), _stream())
+    if rc != 0:
+        raise RuntimeError(f"kx_probe_stream_read failed with HIP error {rc}")
 
 
 def _check(code):

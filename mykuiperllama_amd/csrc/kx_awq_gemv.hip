@@ -190,6 +190,13 @@ inline int check_awq_weights(const int32_t* qweight, const uint16_t* scales, con
     return KX_OK;
 }
 
+// Do the byte ranges [a, a + abytes) and [b, b + bbytes) share a byte?  Null pointers overlap nothing.
+inline bool ranges_overlap(const void* a, size_t abytes, const void* b, size_t bbytes) {
+    if (!a || !b || abytes == 0 || bbytes == 0) return false;
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + bbytes && b0 < a0 + abytes;
+}
+
 // Splits the workspace into counters and partial sums when the plan shares column tiles.
 inline int resolve_workspace(const AwqPlan& p, int M, int N, void* workspace, size_t workspace_bytes,
                              float** partials, uint32_t** counters) {
@@ -395,8 +402,15 @@ extern "C" int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t
         reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
         return KX_ERR_ALIGNMENT;
     }
-    // every workgroup reads the whole incoming row while the first column tile writes the outgoing one
-    if (residual_out == residual || (residual_out && residual_out == delta)) return KX_ERR_ALIAS;
+    // every workgroup reads the whole incoming rows while the first column tile writes the outgoing ones
+    {
+        const size_t row_bytes = static_cast<size_t>(M) * K * sizeof(uint16_t);
+        if (kx::ranges_overlap(residual_out, row_bytes, residual, row_bytes) ||
+            kx::ranges_overlap(residual_out, row_bytes, delta, row_bytes) ||
+            kx::ranges_overlap(residual_out, row_bytes, gain, static_cast<size_t>(K) * sizeof(uint16_t))) {
+            return KX_ERR_ALIAS;
+        }
+    }
     const kx::AwqPlan p = kx::make_fused_plan(M, K, N, false);
     // a thread holds kNormChunks 16-byte pieces of the row for the sum of squares
     if ((K >> 3) > kx::kNormChunks * p.waves * kx::kWave) return KX_ERR_BAD_SHAPE;
@@ -445,7 +459,14 @@ extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_
         reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
         return KX_ERR_ALIGNMENT;
     }
-    if (residual_out == residual || (residual_out && residual_out == delta)) return KX_ERR_ALIAS;
+    {
+        const size_t row_bytes = static_cast<size_t>(K) * sizeof(uint16_t);
+        if (kx::ranges_overlap(residual_out, row_bytes, residual, row_bytes) ||
+            kx::ranges_overlap(residual_out, row_bytes, delta, row_bytes) ||
+            kx::ranges_overlap(residual_out, row_bytes, gain, row_bytes)) {
+            return KX_ERR_ALIAS;
+        }
+    }
     const kx::AwqPlan p = kx::make_fused_plan(1, K, N, false);
     if ((K >> 3) > kx::kNormChunks * p.waves * kx::kWave) return KX_ERR_BAD_SHAPE;
     float* partials = nullptr;
@@ -613,8 +634,23 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
                 reinterpret_cast<uintptr_t>(d->sumsq_out) % 4) {
                 return KX_ERR_ALIGNMENT;
             }
-            // the norm prologue reads all of its row while this epilogue would be rewriting it
-            if (d->in_kind == KX_IN_NORM && d->residual_out == d->norm_row) return KX_ERR_ALIAS;
+            {
+                // Workgroups of other column tiles still read the activations while the tile that finishes
+                // first already writes its 256 columns of the outgoing row: the two must not share a byte.
+                // (residual_out may be residual_in itself: a column is read and written by one thread.)
+                const size_t out_bytes = static_cast<size_t>(N) * sizeof(uint16_t);
+                const size_t in_bytes = static_cast<size_t>(K) * sizeof(uint16_t);
+                if (kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_NORM ? d->norm_row : nullptr, in_bytes) ||
+                    kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_ROW ? d->x : nullptr, in_bytes) ||
+                    kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_SWIGLU ? d->gate : nullptr, in_bytes) ||
+                    kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_SWIGLU ? d->up : nullptr, in_bytes)) {
+                    return KX_ERR_ALIAS;
+                }
+                if (d->residual_out != d->residual_in &&
+                    kx::ranges_overlap(d->residual_out, out_bytes, d->residual_in, out_bytes)) {
+                    return KX_ERR_ALIAS;  // a shifted overlap: another thread's column would be overwritten
+                }
+            }
             res.in = d->residual_in;
             res.out = d->residual_out;
             res.sumsq = d->sumsq_out;

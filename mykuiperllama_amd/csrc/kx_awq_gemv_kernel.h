@@ -303,6 +303,22 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         // keep the scheduler from sinking loads below the first use of an earlier one
         __builtin_amdgcn_sched_barrier(0);
     }
+#if defined(KX_ABLATE) && KX_ABLATE >= 2
+    if constexpr (!STAGED) {
+        if (ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
+            uint32_t f = zw ^ sraw.x ^ sraw.y ^ sraw.z ^ sraw.w;
+#pragma unroll
+            for (int r = 0; r < RT; r++) f ^= w[r];
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+#pragma unroll
+                for (int r8 = 0; r8 < RT / 8; r8++) f ^= xraw[m][r8].x ^ xraw[m][r8].y ^ xraw[m][r8].z ^ xraw[m][r8].w;
+            }
+            if (f == 0x9E3779B9u) partials[tid] = 1.0f;
+            return;
+        }
+    }
+#endif
 
     if constexpr (MERGE) {
         const int wave_id = tid / kWave;
@@ -328,7 +344,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         lds_barrier();
         if (tid < KB) {
             const float total = (s_mpart[0][tid] + s_mpart[1][tid]) + (s_mpart[2][tid] + s_mpart[3][tid]);
-            const uint16_t xv = f32_to_bf16(total / s_norm[tid / kHeadDim]);
+            const float l = s_norm[tid / kHeadDim];
+            const uint16_t xv = f32_to_bf16(l > 0.0f ? total / l : 0.0f);  // no position to attend to: zeros
             s_x[0][tid] = stager ? xv : static_cast<uint16_t>(0);
         }
         lds_barrier();
@@ -489,6 +506,13 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     }
 
     __shared__ uint32_t s_prev;
+#if defined(KX_ABLATE) && KX_ABLATE >= 1
+    if (ktiles > 1) {  // profiling build: no exchange - every workgroup leaves its partial sums and is done
+        const int col = ct * kTileCols + tid;
+        if (tid < kTileCols && col < N) partials[static_cast<size_t>(kt) * M * N + col] = psum[0];
+        return;
+    }
+#endif
     if constexpr (EPI == kEpiStore) {
         splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
                                   &s_prev);

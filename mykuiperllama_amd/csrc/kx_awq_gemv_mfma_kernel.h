@@ -129,6 +129,21 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         }
     }
     __builtin_amdgcn_sched_barrier(0);
+#if defined(KX_ABLATE) && KX_ABLATE >= 2
+    if (ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
+        uint32_t f = 0;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            f ^= xa[ks].x ^ xa[ks].y ^ xa[ks].z ^ xa[ks].w;
+#pragma unroll
+            for (int r = 0; r < 8; r++) f ^= w[ks][r][0] ^ w[ks][r][1];
+        }
+#pragma unroll
+        for (int wv = 0; wv < WAVES; wv++) f ^= s_bits[wv] ^ z_word[wv];
+        if (f == 0x9E3779B9u) partials[tid] = 1.0f;
+        return;
+    }
+#endif
 
     // ---- matrix products ----
     const bf16x8 ones = as_bf16x8(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
@@ -217,6 +232,12 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         }
     }
 
+#if defined(KX_ABLATE) && KX_ABLATE >= 1
+    if (ktiles > 1) {  // profiling build: no exchange - every workgroup leaves its partial sums and is done
+        if (tid < kTileCols && own_col < N) partials[static_cast<size_t>(kt) * M * N + own_col] = psum[0];
+        return;
+    }
+#endif
     if constexpr (ROWS >= 4) {
         static_assert(WAVES * kWave == kTileCols, "the wide exchange is laid out for 256 threads");
         splitk_exchange_store_wide<ROWS>(psum, M, N, ct, kt, ktiles, partials, counters, y, &s_prev);

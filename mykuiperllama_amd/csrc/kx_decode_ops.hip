@@ -381,7 +381,9 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
     s_part[part][d] = acc;
     __syncthreads();
     if (part == 0) {
-        out[static_cast<size_t>(head) * kHeadDim + d] = f32_to_bf16(((s_part[0][d] + s_part[1][d]) + (s_part[2][d] + s_part[3][d])) / s_norm);
+        // no position to attend to (*pos < 0): zeros rather than 0 / 0
+        const float total = (s_part[0][d] + s_part[1][d]) + (s_part[2][d] + s_part[3][d]);
+        out[static_cast<size_t>(head) * kHeadDim + d] = f32_to_bf16(s_norm > 0.0f ? total / s_norm : 0.0f);
     }
 }
 

@@ -9,10 +9,32 @@
 // invalidate the whole L2 once per workgroup: measured ~0.25 us per workgroup, serialised.)
 // Counters sit on 64-byte lines of their own; packed together they serialise at the memory side
 // (~10 ns per atomic, measured).
+//
+// What the exchange relies on, instruction by instruction (gfx950):
+//   1. a producer's partial sums leave as global stores with the device-scope bit (sc1): they are written
+//      through to memory, past its XCD's L2, and a store is only counted as complete (vmcnt) once that
+//      write-through has been acknowledged;
+//   2. s_waitcnt vmcnt(0) in every wave, then the workgroup barrier: when thread 0 passes the barrier, every
+//      partial sum of its workgroup has been acknowledged by memory;
+//   3. only then thread 0 issues the device-scope atomic increment, which executes at the memory side, the
+//      one place all XCDs share;
+//   4. the workgroup that reads ktiles - 1 back knows that every other workgroup's increment, hence by 2
+//      every other workgroup's partial sums, reached memory before; its read-back uses device-scope loads
+//      (sc1), which do not hit in its own, possibly stale, L1 or L2.
+// The compiler keeps 1-3 in order because the wait and the barrier are explicit and the atomics are not
+// reordered across them (the workgroup-scope release fence in front of the wait pins the stores above it).
+// In the language's memory model this is weaker than a release/acquire pair at agent scope; with such a pair
+// the compiler adds a write-back and invalidation of the whole L2 per workgroup (measured: 3 us more on a
+// 256-workgroup launch, 27 us on 2000 workgroups).  Because the argument is about this chip, other targets
+// are refused below, and tests/test_gpu_exchange_soak.py replays thousands of launches on one workspace.
 #ifndef KX_SPLITK_EXCHANGE_H
 #define KX_SPLITK_EXCHANGE_H
 
 #include "kx_common.h"
+
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "kx_splitk_exchange.h orders its memory operations by gfx950's write-through stores and vmcnt acknowledgements; other targets need release/acquire orderings"
+#endif
 
 namespace kx {
 

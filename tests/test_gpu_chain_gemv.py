@@ -246,5 +246,22 @@ def test_chain_rejects_bad_descriptors(capi, torch):
                  "out_kind": capi.OUT_ROW, "y": y}) == -2                                                # parts != K / 256
     assert code({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": s2, "norm_parts": 2, "norm_gain": x,
                  "out_kind": capi.OUT_RESIDUAL, "residual_in": x, "residual_out": x, "sumsq_out": s2}) == -5
+    # overlap is judged on byte ranges, not on base pointers: an outgoing row that starts inside the activations
+    # (or inside a shifted copy of the incoming residual row) is refused as well
+    big = torch.zeros((1, 2 * K), dtype=torch.bfloat16, device="cuda")
+    inside = big[:, 64:64 + N]
+    r_in = torch.zeros((1, N), dtype=torch.bfloat16, device="cuda")
+    assert code({"in_kind": capi.IN_ROW, "x": big[:, :K], "out_kind": capi.OUT_RESIDUAL, "residual_in": r_in,
+                 "residual_out": inside, "sumsq_out": s2}) == -5
+    assert code({"in_kind": capi.IN_SWIGLU, "gate": big[:, :K], "up": x, "out_kind": capi.OUT_RESIDUAL,
+                 "residual_in": r_in, "residual_out": inside, "sumsq_out": s2}) == -5
+    assert code({"in_kind": capi.IN_SWIGLU, "gate": x, "up": big[:, :K], "out_kind": capi.OUT_RESIDUAL,
+                 "residual_in": r_in, "residual_out": inside, "sumsq_out": s2}) == -5
+    assert code({"in_kind": capi.IN_ROW, "x": x, "out_kind": capi.OUT_RESIDUAL, "residual_in": big[:, :N],
+                 "residual_out": inside, "sumsq_out": s2}) == -5
+    # in place (the same row in and out) stays allowed
+    capi.gemv_awq_chain_bf16({"in_kind": capi.IN_ROW, "x": x, "out_kind": capi.OUT_RESIDUAL, "residual_in": r_in,
+                              "residual_out": r_in, "sumsq_out": s2}, qw, sc, qz, K, N, group, ws)
+    torch.cuda.synchronize()
     assert code({"in_kind": capi.IN_ATTN, "attn_workspace": ws, "attn_workspace_bytes": 16, "n_q_heads": 4,
                  "n_kv_heads": 2, "max_positions": 64, "out_kind": capi.OUT_ROW, "y": y}) == -3
