@@ -13,7 +13,15 @@ Prints one JSON line:  value = algorithmic bytes of a step / time of a step, in 
                 the figure includes the dispatch gap between kernels), against 8 TB/s
   cpu_baseline  the oracle's single-threaded fp32 restatement, timed on this host on a bounded
                 number of passes over the same seven shapes
-  per_shape     each projection shape on its own, cold weights, same event timing
+  per_shape     each projection shape on its own, cold weights, same event timing: median / p10 / p90 of the
+                per-launch time over 20 graph replays of 60 launches, and beside it the streaming floor of the
+                same tensors (a kernel that only reads them, mykuiperllama_amd/probe/kx_stream_probe.hip, same
+                rotation, same replay) with the GEMV's distance to it
+  validated     after the timed region the outputs the last timed step left behind are compared with the CPU
+                oracle (fp64 evaluation rounded to bf16) on the same weight set: relative L2 per shape
+  kernel_variants  the same shapes at M = 1 under each kernel the library holds: the two it chooses from (vector
+                ALU, one-shot MFMA) and the two measured alternatives it keeps selectable (K-loop "stream-K" kernel,
+                wide-load kernel through LDS), microseconds per launch
   small_batch   configs[2]: M in {1, 2, 4, 8, 16} on three shapes, microseconds per launch of the
                 vector-ALU kernel and of the MFMA kernel (cold weights, same event timing)
   decode        configs[3] and configs[4]: tokens/s of a full decode step (Qwen3-8B, Qwen3-32B-shaped)
@@ -33,8 +41,10 @@ ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_p
 METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
 # HBM bytes per launch of the dominant kernel (average over the seven launches of a step) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
-# reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).
+# reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).  Counters cannot be
+# read from inside this process, so the figure is carried over from that profile and named as such.
 TRAFFIC_BYTES_PER_LAUNCH = 15288300
+TRAFFIC_SOURCE = "profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md"
 
 
 def parse_args():
@@ -51,6 +61,10 @@ def parse_args():
     ap.add_argument("--no-decode-32b", action="store_true", help="skip the Qwen3-32B-shaped decode step")
     ap.add_argument("--decode-32b", action="store_true", help="kept for older command lines: the step runs by default")
     ap.add_argument("--decode-steps", type=int, default=60)
+    ap.add_argument("--lib", default=None,
+                    help="time another build of the HIP library (e.g. lib/libkx_hip_ablate1.so from "
+                         "`python -m mykuiperllama_amd.build --ablate 1`); its numbers attribute time, its results "
+                         "are wrong by construction, so validation and the decode steps are skipped")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection workload: one 256 MiB device copy (known traffic, for scaling the "
                          "counters) followed by a few cold launches per projection shape; prints no metric")
@@ -111,6 +125,81 @@ def timed_region(torch, launch_steps, steps, warmup, eager, steps_per_graph):
     return e0.elapsed_time(e1) * 1e-3
 
 
+def replay_times(torch, launch_steps, steps_per_graph, replays):
+    """Per-launch-step microseconds of each of `replays` replays of one captured graph of `steps_per_graph` steps."""
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        launch_steps(0, min(steps_per_graph, 4))
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            launch_steps(0, steps_per_graph)
+        g.replay()
+        side.synchronize()
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+        events[0].record(side)
+        for i in range(replays):
+            g.replay()
+            events[i + 1].record(side)
+        side.synchronize()
+    torch.cuda.synchronize()
+    return [events[i].elapsed_time(events[i + 1]) * 1e3 / steps_per_graph for i in range(replays)]
+
+
+def spread(us):
+    """median / p10 / p90 of a list of per-launch microseconds."""
+    v = sorted(us)
+
+    def q(f):
+        return v[min(len(v) - 1, max(0, int(round(f * (len(v) - 1)))))]
+    return {"us": round(q(0.5), 3), "p10_us": round(q(0.1), 3), "p90_us": round(q(0.9), 3)}
+
+
+def shape_report(torch, capi, synth, K, N, group, tensor_sets, x, y, ws):
+    """One projection shape on its own: the GEMV and the streaming floor over the same cold tensors."""
+    nsets = len(tensor_sets)
+    b = synth.awq_gemv_bytes(1, K, N)
+
+    def launch_gemv(first, count):
+        for s in range(first, first + count):
+            qw, sc, qz = tensor_sets[s % nsets]
+            capi.gemv_awq_bf16(x, qw, sc, qz, y, group, ws)
+
+    def launch_floor(first, count):
+        for s in range(first, first + count):
+            capi.probe_stream_read(tensor_sets[s % nsets])
+
+    rep = spread(replay_times(torch, launch_gemv, 5 * nsets, 20))
+    floor = spread(replay_times(torch, launch_floor, 5 * nsets, 20))
+    rep.update({"GB/s": round(b / rep["us"] / 1e3, 1), "pct_of_8TBps": round(b / rep["us"] / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                "bytes": b, "stream_floor_us": floor["us"], "stream_floor_pct_of_8TBps":
+                round(b / floor["us"] / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                "frac_of_floor": round(floor["us"] / rep["us"], 3)})
+    return rep
+
+
+def validate_outputs(torch, sets, last_set, xs, ys, shapes, group):
+    """The outputs the last timed step left in `ys` against the CPU oracle on the same weight set."""
+    import numpy as np
+    from oracle import oracle
+    out = {}
+    worst = 0.0
+    for n in ORDER:
+        K, N = shapes[n]
+        qw, sc, qz = sets[last_set].t[n]
+        xb = xs[K].cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+        ref64 = oracle.gemv_awq_f64(xb, qw.cpu().numpy(), sc.cpu().contiguous().view(torch.int16).numpy().view(np.uint16),
+                                    qz.cpu().numpy(), group)
+        ref = oracle.bf16_to_f32(oracle.f32_to_bf16(ref64.astype(np.float32))).astype(np.float64)
+        got = ys[n].float().cpu().numpy().astype(np.float64)
+        err = float(np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()))
+        out[n] = float(f"{err:.3e}")
+        worst = max(worst, err)
+    return {"validated": bool(worst <= 1e-3), "tolerance_rel_l2": 1e-3, "weight_set": last_set, "rel_l2": out,
+            "checker": "oracle/kx_oracle.c kxo_gemv_awq_f64 rounded to bf16, outside the timed region"}
+
+
 def cpu_baseline(passes):
     """Single-threaded oracle (fp32 evaluation of w = (q - z) * s) over the seven shapes."""
     import numpy as np
@@ -129,8 +218,9 @@ def cpu_baseline(passes):
     out = {"value": round(step_bytes * passes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
            "ms_per_step": round(dt / passes * 1e3, 2),
            "sample": f"{passes} passes over the seven Qwen3-8B projections at M=1 (seeded inputs), "
-                     f"oracle/kx_oracle.c kxo_gemv_awq_f32, gcc -O3 -march=x86-64-v3, one thread, "
-                     f"host has {os.cpu_count()} logical cpus"}
+                     f"oracle/kx_oracle.c kxo_gemv_awq_f32, gcc -O3 -march=x86-64-v3 (the library is built "
+                     f"where there is no GPU and travels to this host, so it cannot be tuned to this host's CPU "
+                     f"with -march=native), one thread, host has {os.cpu_count()} logical cpus"}
     # the same arithmetic spread over the host's cores (columns split across threads), as a second figure
     threads = min(os.cpu_count() or 1, 16)
     if threads > 1:
@@ -143,6 +233,26 @@ def cpu_baseline(passes):
         out["all_cores"] = {"value": round(step_bytes * mt_passes / dt / 1e9, 4), "unit": "GB/s", "cores": threads,
                             "ms_per_step": round(dt / mt_passes * 1e3, 2),
                             "sample": f"{mt_passes} passes, kxo_gemv_awq_f32_range over {threads} threads"}
+    # configs[0]: the single Qwen3-0.6B q_proj GEMV (M=1, K=1024, N=2048), the case the CPU path is quoted on
+    K0, N0 = synth.QWEN3_0P6B["q_proj"]
+    p0 = synth.make_awq_problem("bench_cpu_config0", 1, K0, N0)
+    b0 = synth.awq_gemv_bytes(1, K0, N0)
+    n0 = max(200, passes * 10)
+    oracle.gemv_awq_f32(p0["x"], p0["qweight"], p0["scales"], p0["qzeros"], p0["group"])
+    t0 = time.perf_counter()
+    for _ in range(n0):
+        oracle.gemv_awq_f32(p0["x"], p0["qweight"], p0["scales"], p0["qzeros"], p0["group"])
+    dt = time.perf_counter() - t0
+    cfg0 = {"workload": "configs[0]: Qwen3-0.6B q_proj 1024->2048, M=1", "bytes": b0, "cores": 1,
+            "us_per_gemv": round(dt / n0 * 1e6, 1), "GB/s": round(b0 * n0 / dt / 1e9, 4), "calls": n0}
+    if threads > 1:
+        t0 = time.perf_counter()
+        for _ in range(n0):
+            oracle.gemv_awq_f32_threads(p0["x"], p0["qweight"], p0["scales"], p0["qzeros"], p0["group"], threads)
+        dt = time.perf_counter() - t0
+        cfg0["all_cores"] = {"cores": threads, "us_per_gemv": round(dt / n0 * 1e6, 1),
+                             "GB/s": round(b0 * n0 / dt / 1e9, 4)}
+    out["config0"] = cfg0
     return out
 
 
@@ -184,7 +294,8 @@ def main():
 
     import torch
     from mykuiperllama_amd import capi, synth
-    capi.load()  # raises if the HIP library is missing: there is no fallback path
+    capi.load(args.lib)  # raises if the HIP library is missing: there is no fallback path
+    profiling_build = args.lib is not None
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
@@ -218,6 +329,13 @@ def main():
         return
 
     seconds = timed_region(torch, launch_steps, args.steps, args.warmup, args.eager, WEIGHT_SETS)
+    # which weight set the last timed step walked over (its outputs are what ys holds now)
+    if args.eager:
+        last_set = (args.warmup + args.steps - 1) % WEIGHT_SETS
+    else:
+        rem = args.steps % WEIGHT_SETS
+        last_set = (rem - 1) if rem else (WEIGHT_SETS - 1)
+    validation = None if profiling_build else validate_outputs(torch, sets, last_set, xs, ys, shapes, group)
     ms_per_step = seconds / args.steps * 1e3
     value = step_bytes / (seconds / args.steps) / 1e9
     launches = args.steps * len(ORDER)
@@ -227,22 +345,14 @@ def main():
 
     per_shape = None
     if not args.no_per_shape:
-        per_shape = {}
+        per_shape = {"protocol": "each shape alone, cold weights (12 rotating sets), 20 replays of a 60-launch HIP graph, "
+                                 "events on the launch stream; us = median per-launch time over the replays; "
+                                 "stream_floor_us = the same for a kernel that only reads the shape's three packed "
+                                 "tensors (mykuiperllama_amd/probe/kx_stream_probe.hip)"}
         for n in ["k_proj", "q_proj", "gate_proj", "down_proj"]:
             K, N = shapes[n]
-            b = synth.awq_gemv_bytes(1, K, N)
-            reps = max(WEIGHT_SETS, 240 // WEIGHT_SETS * WEIGHT_SETS)
-
-            def launch_one(first, count, n=n):
-                for s in range(first, first + count):
-                    qw, sc, qz = sets[s % WEIGHT_SETS].t[n]
-                    capi.gemv_awq_bf16(xs[shapes[n][0]], qw, sc, qz, ys[n], group, ws)
-
-            sec = timed_region(torch, launch_one, reps, WEIGHT_SETS, args.eager, WEIGHT_SETS)
-            us = sec / reps * 1e6
-            per_shape[f"{n} {K}x{N}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
-                                         "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
-                                         "bytes": b}
+            per_shape[f"{n} {K}x{N}"] = shape_report(torch, capi, synth, K, N, group, [st.t[n] for st in sets],
+                                                     xs[K], ys[n], ws)
 
         # The launches a decode step fuses along N, and the launches of the Qwen3-32B-shaped step: same
         # cold-weight protocol, one shape at a time (the largest is 131 MB per copy).
@@ -250,28 +360,43 @@ def main():
                        "32B qkv fused": (5120, 10240), "32B o_proj": (8192, 5120),
                        "32B gate+up fused": (5120, 51200), "32B down_proj": (25600, 5120)}
         for n, (K, N) in more_shapes.items():
-            fsets = [WeightSet(torch, {n: (K, N)}, group, gen) for _ in range(WEIGHT_SETS)]
-            b = synth.awq_gemv_bytes(1, K, N)
+            fsets = [WeightSet(torch, {n: (K, N)}, group, gen).t[n] for _ in range(WEIGHT_SETS)]
             xf = xs[K] if K in xs else torch.randn((1, K), device="cuda", generator=gen).bfloat16()
             yf = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
             wsf = capi.make_workspace(1, K, N)
-            reps = 240 // WEIGHT_SETS * WEIGHT_SETS
+            per_shape[f"{n} {K}x{N}"] = shape_report(torch, capi, synth, K, N, group, fsets, xf, yf, wsf)
+            del fsets
+            torch.cuda.empty_cache()
 
-            def launch_f(first, count, n=n, xf=xf, yf=yf, wsf=wsf, fsets=fsets):
-                for s in range(first, first + count):
-                    qw, sc, qz = fsets[s % WEIGHT_SETS].t[n]
-                    capi.gemv_awq_bf16(xf, qw, sc, qz, yf, group, wsf)
+    kernel_variants = None
+    if not args.no_per_shape and not profiling_build:
+        kernel_variants = {"unit": "us per launch, M = 1, cold weights, median of 10 replays of a 60-launch graph",
+                           "kernels": {"vector": "policy 1", "mfma": "policy 2 (one-shot MFMA)",
+                                       "stream": "policy 3 (resident workgroups, K loop)",
+                                       "wide": "policy 4 (16-byte cooperative loads through LDS)"}}
+        for label, (K, N) in {"q_proj": (4096, 4096), "gate_proj": (4096, 12288), "gate+up fused": (4096, 24576),
+                              "32B down_proj": (25600, 5120), "32B gate+up fused": (5120, 51200)}.items():
+            vsets = [WeightSet(torch, {label: (K, N)}, group, gen).t[label] for _ in range(WEIGHT_SETS)]
+            xv = xs[K] if K in xs else torch.randn((1, K), device="cuda", generator=gen).bfloat16()
+            yv = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
+            wsv = capi.make_workspace(1, K, N)
+            row = {}
+            for name, policy in (("vector", 1), ("mfma", 2), ("stream", 3), ("wide", 4)):
+                capi.set_awq_kernel_policy(policy)
 
-            sec = timed_region(torch, launch_f, reps, WEIGHT_SETS, args.eager, WEIGHT_SETS)
-            us = sec / reps * 1e6
-            per_shape[f"{n} {K}x{N}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
-                                         "pct_of_8TBps": round(b / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
-                                         "bytes": b}
-            del fsets, launch_f
+                def launch_v(first, count, vsets=vsets, xv=xv, yv=yv, wsv=wsv):
+                    for s_ in range(first, first + count):
+                        qw, sc, qz = vsets[s_ % WEIGHT_SETS]
+                        capi.gemv_awq_bf16(xv, qw, sc, qz, yv, group, wsv)
+
+                row[name] = spread(replay_times(torch, launch_v, 5 * WEIGHT_SETS, 10))["us"]
+            capi.set_awq_kernel_policy(0)
+            kernel_variants[f"{label} {K}x{N}"] = row
+            del vsets
             torch.cuda.empty_cache()
 
     small_batch = None
-    if not args.no_small_batch:
+    if not args.no_small_batch and not profiling_build:
         small_batch = {"unit": "us per launch", "kernels": {"vector": "VALU kernel, bf16 dot2", "mfma": "16x16x32 bf16 MFMA"}}
         for n in ["q_proj", "gate_proj", "down_proj"]:
             K, N = shapes[n]
@@ -313,19 +438,29 @@ def main():
         "config": {"workload": "configs[1]: the seven Qwen3-8B decoder projections at M=1, INT4 AWQ group 128, "
                                f"cold weights ({WEIGHT_SETS} rotating sets, {WEIGHT_SETS * step_bytes / 1e9:.2f} GB)",
                    "launch": "eager" if args.eager else "hipGraph replay",
-                   "bytes_per_step": step_bytes, "launches_per_step": len(ORDER)},
+                   "bytes_per_step": step_bytes, "launches_per_step": len(ORDER),
+                   "weights": f"torch.randint / torch.rand on the device, torch.Generator(cuda) seeded {synth.BASE_SEED} "
+                              "(uniform int4 codes and zero points, fp16 scales U(0.001, 0.02)), activations "
+                              "bf16 N(0,1) from the same generator",
+                   "library": args.lib or "mykuiperllama_amd/lib/libkx_hip.so"},
         "pct_of_8TBps": round(value / HBM_PEAK_GBPS * 100, 2),
         "decode_tok_s": None,
         "roofline": {"bound": "hbm", "kernel": "kx::awq_gemv_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": round(bytes_per_launch),
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "traffic_source": TRAFFIC_SOURCE,
+                     "bytes_per_launch": round(bytes_per_launch),
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
+    if validation is not None:
+        out["validated"] = validation["validated"]
+        out["validation"] = validation
     if per_shape is not None:
         out["per_shape"] = per_shape
+    if kernel_variants is not None:
+        out["kernel_variants"] = kernel_variants
     if small_batch is not None:
         out["small_batch"] = small_batch
-    if not args.no_decode:
+    if not args.no_decode and not profiling_build:
         del sets
         torch.cuda.empty_cache()
         d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager)

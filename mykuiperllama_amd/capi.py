@@ -222,11 +222,11 @@ _policy = 0
 def set_awq_kernel_policy(policy):
     """Test and benchmark plumbing: which kernel gemv_awq_bf16 of THIS module asks for from now on.
     0 = the product entry point (the library chooses by shape); 1 = vector-ALU kernel, 2 = one-shot MFMA
-    kernel, each through the internal entry point kx_gemv_awq_bf16_policy.
+    kernel, 3 / 4 = the two measured alternatives (K-loop kernel, wide-load kernel), each through the internal entry point kx_gemv_awq_bf16_policy.
     The library itself keeps no such state."""
     global _policy
-    if policy not in (0, 1, 2):
-        raise ValueError("policy must be 0, 1 or 2")
+    if policy not in (0, 1, 2, 3, 4):
+        raise ValueError("policy must be 0 .. 4")
     _policy = policy
 
 
