@@ -219,6 +219,10 @@ typedef struct kx_chain_desc {
     uint16_t* k_cache;
     uint16_t* v_cache;
     const int32_t* pos;
+    /* activation rows (0 reads as 1) and, for KX_IN_SWIGLU / KX_IN_NORM, the elements between
+     * consecutive rows of gate / up / norm_row (0 reads as K) */
+    int32_t rows;
+    int32_t act_ld;
 } kx_chain_desc;
 
 int kx_gemv_awq_chain_bf16(const kx_chain_desc* desc, const int32_t* qweight, const uint16_t* scales,

@@ -109,7 +109,7 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
 inline AwqPlan make_plan(int M, int K, int N, int group, int mode) {
     // The MFMA kernel needs quantisation groups that tile the workgroup's K range (powers of two)
     // and loads two packed words at a time (N a multiple of sixteen).
-    const bool mfma_ok = is_pow2(group) && (N % 16) == 0;
+    const bool mfma_ok = is_pow2(group) && (N % 16) == 0;  // mfma_shape_ok() below
     // One activation row stays on the vector kernel although the MFMA kernel is a few per cent faster on
     // wide projections (us per launch, vector / MFMA: 4096->12288 8.9 / 8.5, 4096->24576 13.5 / 13.0,
     // 5120->51200 30.9 / 29.3; narrow and tall ones the other way round: 4096->4096 5.7 / 5.8, 12288->4096
@@ -250,6 +250,38 @@ void launch_fused(const AwqPlan& p, const FusedInput& fi, const int32_t* qweight
     else KX_BY_MB(4, 8);
 #undef KX_BY_MB
 #undef KX_ARGS
+}
+
+// The matrix-core kernel with an activation prologue and / or the residual epilogue, 2 <= M <= 16.
+template <int PRO, int EPI>
+void launch_mfma_fused(const AwqPlan& p, const FusedInput& fi, const ResidualTarget& res, const uint16_t* x,
+                       const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros, uint16_t* y,
+                       float* partials, uint32_t* counters, int M, int K, int N, int group, hipStream_t stream) {
+    int group_shift = 0;
+    while ((1 << group_shift) < group) group_shift++;
+#define KX_MARGS x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_shift, p.coltiles, p.ktiles, stream, fi, res
+#define KX_MFMA_BY_M(KS)                                                             \
+    do {                                                                             \
+        if (M <= 2) launch_awq_gemv_mfma<4, KS, 2, 1, PRO, EPI>(KX_MARGS);           \
+        else if (M <= 4) launch_awq_gemv_mfma<4, KS, 4, 1, PRO, EPI>(KX_MARGS);      \
+        else if (M <= 8) launch_awq_gemv_mfma<4, KS, 8, 1, PRO, EPI>(KX_MARGS);      \
+        else launch_awq_gemv_mfma<4, KS, 8, 2, PRO, EPI>(KX_MARGS);                  \
+    } while (0)
+    if (p.rt == 4) KX_MFMA_BY_M(4);
+    else if (p.rt == 2) KX_MFMA_BY_M(2);
+    else KX_MFMA_BY_M(1);
+#undef KX_MFMA_BY_M
+#undef KX_MARGS
+}
+
+// What the matrix-core kernel asks of a shape: quantisation groups that tile the workgroup's K range
+// (powers of two) and two packed words per load (N a multiple of sixteen).
+inline bool mfma_shape_ok(int N, int group) {
+    return is_pow2(group) && (N % 16) == 0;
+}
+
+inline bool aligned_to(const void* p, size_t a) {
+    return reinterpret_cast<uintptr_t>(p) % a == 0;
 }
 
 // Checks shared by every AWQ entry point; `x` stands for whichever tensors feed the activations.
@@ -517,15 +549,28 @@ extern "C" int kx_gemv_awq_swiglu_bf16(const uint16_t* gate, const uint16_t* up,
     if (rc != KX_OK) return rc;
     if (act_ld < K) return KX_ERR_BAD_SHAPE;
     if (reinterpret_cast<uintptr_t>(gate) % 2 || reinterpret_cast<uintptr_t>(up) % 2) return KX_ERR_ALIGNMENT;
+    kx::FusedInput fi{};
+    fi.a = gate;
+    fi.b = up;
+    fi.ld = act_ld;
+    // Several rows go to the matrix cores, as in kx_gemv_awq_bf16, when gate and up can be read 16 bytes at a time
+    if (M >= 2 && kx::mfma_shape_ok(N, group_size) && kx::aligned_to(gate, 16) && kx::aligned_to(up, 16) &&
+        (act_ld % 8) == 0) {
+        const kx::AwqPlan mp = kx::make_mfma_plan(M, K, N, group_size);
+        float* partials = nullptr;
+        uint32_t* counters = nullptr;
+        rc = kx::resolve_workspace(mp, M, N, workspace, workspace_bytes, &partials, &counters);
+        if (rc != KX_OK) return rc;
+        kx::launch_mfma_fused<kx::kProSwiGLU, kx::kEpiStore>(mp, fi, kx::ResidualTarget{}, nullptr, qweight, scales,
+                                                             qzeros, y, partials, counters, M, K, N, group_size,
+                                                             kx::as_stream(stream));
+        return kx::launch_status();
+    }
     const kx::AwqPlan p = kx::make_fused_plan(M, K, N, true);
     float* partials = nullptr;
     uint32_t* counters = nullptr;
     rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
     if (rc != KX_OK) return rc;
-    kx::FusedInput fi{};
-    fi.a = gate;
-    fi.b = up;
-    fi.ld = act_ld;
     kx::launch_fused<kx::kProSwiGLU>(p, fi, qweight, scales, qzeros, y, partials, counters, M, K, N, group_size,
                                      kx::as_stream(stream));
     return kx::launch_status();
@@ -711,6 +756,15 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
     const uint16_t* x = nullptr;
     uint16_t* y = nullptr;
     bool long_rows = true;
+    const int rows = d->rows > 0 ? d->rows : 1;
+    if (rows > KX_MAX_BATCH || K < 1 || N < 8) return KX_ERR_BAD_SHAPE;
+    const int act_ld = d->act_ld > 0 ? d->act_ld : K;
+    if (act_ld < K) return KX_ERR_BAD_SHAPE;
+    if (rows > 1) {
+        // several rows: the matrix-core kernel, which produces activations 16 bytes at a time
+        if (d->in_kind == KX_IN_ATTN || d->out_kind == KX_OUT_QKV_ROPE) return KX_ERR_BAD_SHAPE;
+        if (!kx::mfma_shape_ok(N, group_size) || (act_ld % 8) != 0) return KX_ERR_BAD_SHAPE;
+    }
 
     // where the activations come from
     switch (d->in_kind) {
@@ -722,9 +776,10 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
         case KX_IN_SWIGLU:
             if (!d->gate || !d->up) return KX_ERR_NULL_POINTER;
             if (reinterpret_cast<uintptr_t>(d->gate) % 2 || reinterpret_cast<uintptr_t>(d->up) % 2) return KX_ERR_ALIGNMENT;
+            if (rows > 1 && (!kx::aligned_to(d->gate, 16) || !kx::aligned_to(d->up, 16))) return KX_ERR_ALIGNMENT;
             fi.a = d->gate;
             fi.b = d->up;
-            fi.ld = K;
+            fi.ld = act_ld;
             break;
         case KX_IN_ATTN: {
             if (!d->attn_workspace) return KX_ERR_NULL_POINTER;
@@ -751,12 +806,13 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
                 reinterpret_cast<uintptr_t>(d->norm_gain) % 2) {
                 return KX_ERR_ALIGNMENT;
             }
+            if (rows > 1 && (!kx::aligned_to(d->norm_row, 16) || !kx::aligned_to(d->norm_gain, 16))) return KX_ERR_ALIGNMENT;
             fi.a = d->norm_row;
             fi.gain = d->norm_gain;
             fi.eps = d->norm_eps;
             fi.sumsq = d->norm_sumsq;
             fi.sumsq_parts = d->norm_parts;
-            fi.ld = K;
+            fi.ld = act_ld;
             break;
         default: return KX_ERR_BAD_SHAPE;
     }
@@ -779,8 +835,8 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
                 // Workgroups of other column tiles still read the activations while the tile that finishes
                 // first already writes its 256 columns of the outgoing row: the two must not share a byte.
                 // (residual_out may be residual_in itself: a column is read and written by one thread.)
-                const size_t out_bytes = static_cast<size_t>(N) * sizeof(uint16_t);
-                const size_t in_bytes = static_cast<size_t>(K) * sizeof(uint16_t);
+                const size_t out_bytes = static_cast<size_t>(rows) * N * sizeof(uint16_t);
+                const size_t in_bytes = (static_cast<size_t>(rows - 1) * act_ld + K) * sizeof(uint16_t);
                 if (kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_NORM ? d->norm_row : nullptr, in_bytes) ||
                     kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_ROW ? d->x : nullptr, in_bytes) ||
                     kx::ranges_overlap(d->residual_out, out_bytes, d->in_kind == KX_IN_SWIGLU ? d->gate : nullptr, in_bytes) ||
@@ -811,9 +867,32 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
         default: return KX_ERR_BAD_SHAPE;
     }
     // 8-byte alignment is what the plain store asks of y; the other outputs are written per element
-    int rc = kx::check_awq_weights(qweight, scales, qzeros, out_probe, 1, K, N, group_size, d->out_kind == KX_OUT_ROW);
+    int rc = kx::check_awq_weights(qweight, scales, qzeros, out_probe, rows, K, N, group_size, d->out_kind == KX_OUT_ROW);
     if (rc != KX_OK) return rc;
     if (d->in_kind == KX_IN_ATTN && (K % kx::kHeadDim) != 0) return KX_ERR_BAD_SHAPE;
+
+    if (rows > 1) {
+        const kx::AwqPlan mp = kx::make_mfma_plan(rows, K, N, group_size);
+        float* partials = nullptr;
+        uint32_t* counters = nullptr;
+        rc = kx::resolve_workspace(mp, rows, N, workspace, workspace_bytes, &partials, &counters);
+        if (rc != KX_OK) return rc;
+        hipStream_t s = kx::as_stream(stream);
+#define KX_MCHAIN(PRO, EPI) kx::launch_mfma_fused<PRO, EPI>(mp, fi, res, x, qweight, scales, qzeros, y, partials, counters, rows, K, N, group_size, s)
+#define KX_MBY_OUT(PRO)                                                       \
+    do {                                                                      \
+        if (d->out_kind == KX_OUT_ROW) KX_MCHAIN(PRO, kx::kEpiStore);         \
+        else KX_MCHAIN(PRO, kx::kEpiResidual);                                \
+    } while (0)
+        switch (d->in_kind) {
+            case KX_IN_ROW: KX_MBY_OUT(kx::kProNone); break;
+            case KX_IN_SWIGLU: KX_MBY_OUT(kx::kProSwiGLU); break;
+            default: KX_MBY_OUT(kx::kProPreNorm); break;
+        }
+#undef KX_MBY_OUT
+#undef KX_MCHAIN
+        return kx::launch_status();
+    }
 
     const bool plain_ends = (d->in_kind == KX_IN_ROW || d->in_kind == KX_IN_SWIGLU) &&
                             (d->out_kind == KX_OUT_ROW || d->out_kind == KX_OUT_RESIDUAL);

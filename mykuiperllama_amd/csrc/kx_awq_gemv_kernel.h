@@ -24,6 +24,7 @@
 
 #include "kx_attn_merge.h"
 #include "kx_common.h"
+#include "kx_gemv_fused.h"
 #include "kx_rope.h"
 #include "kx_splitk_exchange.h"
 
@@ -60,46 +61,6 @@ __device__ __forceinline__ void unpack_codes(uint32_t w, float (&q)[8]) {
     q[order_of(7)] = d.y;
 }
 
-// Activations may be produced on the way in instead of being read as a finished bf16 row
-// (PRO below); the producing arithmetic and its rounding points are those of the stand-alone
-// kernels, so a fused launch returns what the separate launches would.
-constexpr int kProNone = 0;     // x is a bf16 [M, K] tensor
-constexpr int kProSwiGLU = 1;   // x[m,k] = bf16( bf16(silu(a[m,k])) * b[m,k] )
-constexpr int kProAddNorm = 2;  // r = bf16(a + b) (b optional), x = gain * bf16(r * rsqrt(mean(r^2) + eps))
-constexpr int kProAddNormLong = 3;  // the same for rows of more than eight elements per thread
-constexpr int kProAttnMerge = 4;  // x = the attention output, merged here from the per-chunk results (M = 1)
-constexpr int kProPreNorm = 5;    // x = gain * bf16(a * rsqrt(mean(a^2) + eps)), the sum of squares given per 256 columns (M = 1)
-constexpr int kNormChunks = 2;  // most 16-byte pieces of a row a thread holds for the sum of squares
-constexpr int kMergeHold = 20;  // per-chunk values a thread holds per element it merges: 80 chunks in four parts
-constexpr int kMergeStatsPerLane = 2;  // chunks per lane of the wave that prepares a head's factors (>= 80 / 64)
-
-struct FusedInput {
-    const uint16_t* a;     // gate, or the residual stream
-    const uint16_t* b;     // up, or the delta to add to the residual stream (may be null)
-    const uint16_t* gain;  // norm gain [K]
-    uint16_t* r_out;       // where the updated residual stream goes (may be null); must not alias a
-    int ld;                // elements between consecutive activation rows of a and b
-    float eps;
-    // kProAttnMerge: results of the first attention stage (layout in kx_attn_merge.h)
-    const float* part_out;
-    const float* part_ml;
-    int nchunks;
-    int heads_per_kv;
-    // kProPreNorm: sum of squares of row `a`, one partial per tile of 256 columns (at most 64)
-    const float* sumsq;
-    int sumsq_parts;
-};
-
-// kEpiResidual: the finished row o is added to the residual stream, out = bf16(in + bf16(o)), and the
-// sum of squares of the new row is left per column tile for the RMSNorm that follows:
-//   sumsq[t] = ((Q0 + Q1) + Q2) + Q3,  Q_i = wave_sum over the 64 columns of quarter i of tile t
-// (kProPreNorm adds the tiles with one more wave_sum, lane = tile).
-struct ResidualTarget {
-    const uint16_t* in;   // bf16 [N]
-    uint16_t* out;        // bf16 [N], may be `in`: a column is read and written by the same thread
-    float* sumsq;         // [ceil(N / 256)]
-};
-
 constexpr float kCodeOffset = 16.0f;
 
 // Two bf16 16.0 in a register whose value the compiler cannot see, so that (v & mask) | magic
@@ -124,11 +85,6 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     __builtin_memcpy(&vb, &b, 4);
     return __builtin_amdgcn_fdot2_f32_bf16(va, vb, c, false);
 }
-
-// What happens to the finished sums (EPI below).
-constexpr int kEpiStore = 0;   // y[m, n] = bf16(sum)
-constexpr int kEpiQkRope = 1;  // the row is q | k | v heads of 128: per-head norm, rotation, cache append (M = 1)
-constexpr int kEpiResidual = 2;  // residual add + per-tile sums of squares (M = 1), see ResidualTarget
 
 template <int WAVES, int RT, int MB, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(

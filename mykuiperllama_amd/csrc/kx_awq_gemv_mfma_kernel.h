@@ -22,10 +22,16 @@
 //
 // Cost per weight: one VALU operation to build the operand (two byte permutes, three shifts and
 // eight and/or pairs per sixteen weights) and 1/512 of an MFMA, whatever M is.
+//
+// The activations may be produced on the way in (PRO: SwiGLU of two tensors, or an RMSNorm whose sum of
+// squares arrives per 256 columns) and the result may be added to a residual stream on the way out (EPI),
+// with the arithmetic and rounding points of the stand-alone kernels.  A produced activation is staged
+// in LDS as bf16, the workgroup's K range of every row, and the A operand is read from there.
 #ifndef KX_AWQ_GEMV_MFMA_KERNEL_H
 #define KX_AWQ_GEMV_MFMA_KERNEL_H
 
 #include "kx_common.h"
+#include "kx_gemv_fused.h"
 #include "kx_splitk_exchange.h"
 
 namespace kx {
@@ -51,22 +57,50 @@ __device__ __forceinline__ uint32_t code_pair_to_bf16(uint32_t v, uint32_t magic
     return (v & 0x000F000Fu) | magic;
 }
 
+// Eight consecutive bf16 of a 16-byte piece as floats, and back (round to nearest even).
+__device__ __forceinline__ void bf16x8_to_f32(const uint4& v, float (&f)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) f[i] = __uint_as_float((i & 1) ? (w[i >> 1] & 0xffff0000u) : (w[i >> 1] << 16));
+}
+__device__ __forceinline__ uint4 f32_to_bf16x8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        w[i] = static_cast<uint32_t>(f32_to_bf16(f[2 * i])) | (static_cast<uint32_t>(f32_to_bf16(f[2 * i + 1])) << 16);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // KS: consecutive 32-row steps per wave (they must share a quantisation group);
 // MC: activation rows a workgroup reduces per LDS round (1, 2, 4 or 8); ROUNDS: 2 for M > 8, else 1.
-template <int WAVES, int KS, int MC, int ROUNDS>
+// With a prologue, `x` is not read: fi.a / fi.b (/ fi.gain) are 16-byte aligned, fi.ld a multiple of eight.
+template <int WAVES, int KS, int MC, int ROUNDS, int PRO = kProNone, int EPI = kEpiStore>
 __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group_shift, int ktiles) {
+    int M, int K, int N, int group_shift, int ktiles, FusedInput fi, ResidualTarget res) {
     constexpr int WROWS = KS * kStepRows;  // rows of K per wave
     constexpr int KB = WAVES * WROWS;      // rows of K per workgroup
     constexpr int ROWS = MC * ROUNDS;      // activation rows this kernel carries (>= M)
-    static_assert(WAVES * kWave >= kTileCols, "one thread per tile column");
+    constexpr int THREADS = WAVES * kWave;
+    static_assert(THREADS >= kTileCols, "one thread per tile column");
+    static_assert(PRO == kProNone || PRO == kProSwiGLU || PRO == kProPreNorm, "prologues of the matrix-core kernel");
+    static_assert(EPI == kEpiStore || EPI == kEpiResidual, "epilogues of the matrix-core kernel");
+    constexpr bool STAGED = PRO != kProNone;
+    // A staged row is the workgroup's K range plus 16 bytes, so that the rows a wave reads together
+    // start in different banks.
+    constexpr int XPITCH = KB + 8;
+    constexpr int KPIECES = KB / 8;             // 16-byte pieces per staged row
+    constexpr int PIECES = ROWS * KPIECES;
+    constexpr int PPT = (PIECES + THREADS - 1) / THREADS;  // pieces a thread produces
 
     __shared__ __attribute__((aligned(16))) float red[WAVES][MC][kTileCols];
     __shared__ float xs_red[WAVES][MC];
     __shared__ uint32_t s_prev;
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? ROWS : 1][STAGED ? XPITCH : 8];
+    __shared__ float s_inv[PRO == kProPreNorm ? ROWS : 1];
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
@@ -78,6 +112,37 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     const int nw = N >> 3;
 
     const int kwave = kt * KB + wave * WROWS;  // first row of this wave
+
+    // ---- operands of the activation prologue go out first: they are small, mostly cached, and the prologue
+    // should run while the weights are still on their way ----
+    // Piece e = tid + i * THREADS of the workgroup is (row e / KPIECES, elements 8 (e % KPIECES) .. + 7 of
+    // the K range); addresses are clamped, what a clamped load brings is replaced by zeros.
+    uint4 pa[STAGED ? PPT : 1], pb[STAGED ? PPT : 1];
+    float tile_ss[PRO == kProPreNorm ? (ROWS + WAVES - 1) / WAVES : 1];
+    if constexpr (STAGED) {
+#pragma unroll
+        for (int i = 0; i < PPT; i++) {
+            const int e = tid + i * THREADS;
+            const int pm = e / KPIECES;
+            const int k = kt * KB + 8 * (e % KPIECES);
+            const int mc = pm < M ? pm : M - 1;
+            const int kc = k < K ? k : K - 8;
+            const size_t at = static_cast<size_t>(mc) * fi.ld + kc;
+            pa[i] = *reinterpret_cast<const uint4*>(fi.a + at);
+            if constexpr (PRO == kProSwiGLU) pb[i] = *reinterpret_cast<const uint4*>(fi.b + at);
+            else pb[i] = *reinterpret_cast<const uint4*>(fi.gain + kc);
+        }
+        if constexpr (PRO == kProPreNorm) {
+            // wave w adds the tiles of rows w, w + WAVES, ...: lane = tile
+#pragma unroll
+            for (int rr = 0; rr < (ROWS + WAVES - 1) / WAVES; rr++) {
+                const int m = wave + rr * WAVES;
+                const int mc = m < M ? m : M - 1;
+                tile_ss[rr] = fi.sumsq[static_cast<size_t>(mc) * fi.sumsq_parts +
+                                       (lane < fi.sumsq_parts ? lane : fi.sumsq_parts - 1)];
+            }
+        }
+    }
 
     // ---- loads, all issued before anything is consumed ----
     // Every load is unconditional: an address that would fall outside is clamped to one inside, and
@@ -103,13 +168,15 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     // past M and steps past K (K is a multiple of 32: a step is all in or all out) are zeros.
     uint4 xa[KS];
     const int x_row = c < M ? c : M - 1;
+    if constexpr (!STAGED) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-        const int kstep = kwave + ks * kStepRows;
-        const int kld = kstep < K ? kstep : K - kStepRows;
-        const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(x_row) * K + kld + 8 * b);
-        const bool live = c < M && kstep < K;
-        xa[ks] = make_uint4(live ? got.x : 0u, live ? got.y : 0u, live ? got.z : 0u, live ? got.w : 0u);
+        for (int ks = 0; ks < KS; ks++) {
+            const int kstep = kwave + ks * kStepRows;
+            const int kld = kstep < K ? kstep : K - kStepRows;
+            const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(x_row) * K + kld + 8 * b);
+            const bool live = c < M && kstep < K;
+            xa[ks] = make_uint4(live ? got.x : 0u, live ? got.y : 0u, live ? got.z : 0u, live ? got.w : 0u);
+        }
     }
     // The lane's two word columns, eight rows per step, both words in one load: the host sends only
     // N that are multiples of sixteen here, so word rows are 8-byte aligned.
@@ -130,7 +197,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
 #if defined(KX_ABLATE) && KX_ABLATE >= 2
-    if (ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
+    if (!STAGED && ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
         uint32_t f = 0;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
@@ -144,6 +211,53 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         return;
     }
 #endif
+
+    // ---- the activation prologue: produce the staged rows, then read the A operand back ----
+    if constexpr (STAGED) {
+        if constexpr (PRO == kProPreNorm) {
+#pragma unroll
+            for (int rr = 0; rr < (ROWS + WAVES - 1) / WAVES; rr++) {
+                const int m = wave + rr * WAVES;
+                const float total = wave_sum(lane < fi.sumsq_parts ? tile_ss[rr] : 0.0f);
+                if (lane == 0 && m < ROWS) s_inv[m] = 1.0f / sqrtf(total / static_cast<float>(K) + fi.eps);
+            }
+            lds_barrier();
+        }
+#pragma unroll
+        for (int i = 0; i < PPT; i++) {
+            const int e = tid + i * THREADS;
+            const int pm = e / KPIECES;
+            const int kp = e % KPIECES;
+            if (pm < ROWS) {
+                float av[8], bv[8], out[8];
+                bf16x8_to_f32(pa[i], av);
+                bf16x8_to_f32(pb[i], bv);
+                const bool live = pm < M && kt * KB + 8 * kp < K;  // K is a multiple of eight: a piece is all in or all out
+                if constexpr (PRO == kProSwiGLU) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const float act = bf16_to_f32(f32_to_bf16(av[j] / (1.0f + expf(-av[j]))));
+                        out[j] = live ? act * bv[j] : 0.0f;
+                    }
+                } else {
+                    const float inv = s_inv[pm];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        out[j] = live ? bv[j] * bf16_to_f32(f32_to_bf16(av[j] * inv)) : 0.0f;
+                    }
+                }
+                *reinterpret_cast<uint4*>(&s_x[pm][8 * kp]) = f32_to_bf16x8(out);
+            }
+        }
+        lds_barrier();
+        const int s_row = c < ROWS ? c : ROWS - 1;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const uint4 got = *reinterpret_cast<const uint4*>(&s_x[s_row][(wave * KS + ks) * kStepRows + 8 * b]);
+            const bool live = c < M;  // rows M .. ROWS-1 and elements past K were staged as zeros
+            xa[ks] = make_uint4(live ? got.x : 0u, live ? got.y : 0u, live ? got.z : 0u, live ? got.w : 0u);
+        }
+    }
 
     // ---- matrix products ----
     const bf16x8 ones = as_bf16x8(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
@@ -238,25 +352,54 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         return;
     }
 #endif
-    if constexpr (ROWS >= 4) {
-        static_assert(WAVES * kWave == kTileCols, "the wide exchange is laid out for 256 threads");
+    if constexpr (EPI == kEpiResidual) {
+        static_assert(THREADS == kTileCols, "the residual epilogue is laid out for 256 threads");
+        float sum[ROWS];
+        if (!splitk_exchange_sum<ROWS>(psum, sum, 0, M, N, ct, kt, ktiles, ct, partials, counters, &s_prev)) return;
+        __shared__ float s_quarter[ROWS][kTileCols / kWave];
+        const bool col_ok = own_col < N;
+        uint16_t rin[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            rin[r] = res.in[static_cast<size_t>(r < M ? r : M - 1) * N + own_ld];
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            float rv = 0.0f;
+            if (col_ok && r < M) {
+                const float o = bf16_to_f32(f32_to_bf16(sum[r]));  // the projection's output is a bf16 tensor
+                const uint16_t rbits = f32_to_bf16(bf16_to_f32(rin[r]) + o);
+                res.out[static_cast<size_t>(r) * N + own_col] = rbits;
+                rv = bf16_to_f32(rbits);
+            }
+            const float q = wave_sum(rv * rv);
+            if (lane == 0) s_quarter[r][wave] = q;
+        }
+        __syncthreads();
+        if (tid < M) {
+            res.sumsq[static_cast<size_t>(tid) * gridDim.x + ct] =
+                ((s_quarter[tid][0] + s_quarter[tid][1]) + s_quarter[tid][2]) + s_quarter[tid][3];
+        }
+    } else if constexpr (ROWS >= 4) {
+        static_assert(THREADS == kTileCols, "the wide exchange is laid out for 256 threads");
         splitk_exchange_store_wide<ROWS>(psum, M, N, ct, kt, ktiles, partials, counters, y, &s_prev);
     } else {
         splitk_exchange_store<ROWS>(psum, 0, M, N, ct, kt, ktiles, ct, partials, counters, y, &s_prev);
     }
 }
 
-template <int WAVES, int KS, int MC, int ROUNDS>
+template <int WAVES, int KS, int MC, int ROUNDS, int PRO = kProNone, int EPI = kEpiStore>
 inline void launch_awq_gemv_mfma(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,
                                  const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
                                  int M, int K, int N, int group_shift, int coltiles, int ktiles,
-                                 hipStream_t stream) {
+                                 hipStream_t stream, const FusedInput& fi = FusedInput{},
+                                 const ResidualTarget& res = ResidualTarget{}) {
     dim3 grid(coltiles, ktiles, 1);
     dim3 block(WAVES * kWave, 1, 1);
-    hipLaunchKernelGGL((awq_gemv_mfma_kernel<WAVES, KS, MC, ROUNDS>), grid, block, 0, stream, x,
+    hipLaunchKernelGGL((awq_gemv_mfma_kernel<WAVES, KS, MC, ROUNDS, PRO, EPI>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group_shift, ktiles);
+                       group_shift, ktiles, fi, res);
 }
 
 }  // namespace kx

@@ -2,7 +2,7 @@
 #include "kx_common.h"
 
 extern "C" int kx_abi_version(void) {
-    return 2;
+    return 3;
 }
 
 extern "C" const char* kx_error_string(int code) {

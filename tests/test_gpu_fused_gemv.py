@@ -86,6 +86,8 @@ def test_swiglu_prologue_equals_separate_launches(capi, torch, oracle, M, K, N, 
     y_sep = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     y_fused = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     capi.swiglu_bf16(gate.contiguous(), up.contiguous(), act)
+    # several rows: the fused launch runs on the kernel the plain entry point picks by shape
+    capi.set_awq_kernel_policy(1 if M == 1 else 0)
     capi.gemv_awq_bf16(act, qw, sc, qz, y_sep, group, ws)
     capi.gemv_awq_swiglu_bf16(gate, up, qw, sc, qz, y_fused, group, ws)
     torch.cuda.synchronize()
