@@ -256,7 +256,7 @@ def cpu_baseline(passes):
     return out
 
 
-def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager):
+def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager, batches=()):
     """Tokens/s of a full random-init decode step (batch 1, KV cache pre-filled at `ctx`)."""
     from mykuiperllama_amd import decode
     cfg = {"qwen3-8b": decode.QWEN3_8B, "qwen3-32b": decode.QWEN3_32B}[cfg_name]
@@ -280,6 +280,29 @@ def decode_benchmark(torch, cfg_name, ctx, steps, warmup, eager):
                     "launches_per_token": model.launches_per_step(with_head)}
     torch.cuda.synchronize()
     out["next_token_finite"] = bool(torch.isfinite(model.logits.float()).all().item())
+    if batches:
+        # several sequences decoded together, every one of them at position `ctx` of its own cache: the GEMVs
+        # read the weights once for all rows, the attention reads one cache per sequence
+        rows = {}
+        for B in batches:
+            bm = decode.BatchDecodeModel(model, B)
+            bm.prefill_cache_random(ctx)
+            bm.set_input([1 + b for b in range(B)], [ctx] * B)
+            cell = {}
+            for label, fused in (("fused", True), ("unfused", False)):
+                def launch(first, count, fused=fused):
+                    for _ in range(count):
+                        bm.step(fused=fused)
+                n = max(8, steps // 3)
+                sec = timed_region(torch, launch, n, 4, eager, 4)
+                cell[label] = {"ms_per_step": round(sec / n * 1e3, 4), "tokens_per_s": round(B * n / sec, 1),
+                               "launches_per_step": bm.launches_per_step(True, fused)}
+            torch.cuda.synchronize()
+            cell["finite"] = bool(torch.isfinite(bm.logits.float()).all().item())
+            rows[f"B={B}"] = cell
+            del bm
+            torch.cuda.empty_cache()
+        out["small_batch_decode"] = rows
     del model
     torch.cuda.empty_cache()
     return out
@@ -465,7 +488,7 @@ def main():
     if not args.no_decode and not profiling_build:
         del sets
         torch.cuda.empty_cache()
-        d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager)
+        d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager, batches=(2, 8, 16))
         out["decode_tok_s"] = d8["with_lm_head"]["tokens_per_s"]
         out["decode"] = {"qwen3-8b ctx4096": d8}
         if not args.no_decode_32b:

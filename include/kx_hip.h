@@ -145,8 +145,8 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
                               int32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
- * Chained GEMV (M = 1): one launch whose activations come from the previous operator of a decoder
- * layer and whose result goes straight into the next one.  `in_kind` selects where the activation
+ * Chained GEMV: one launch whose activations come from the previous operator of a decoder
+ * layer and whose result goes straight into the next one.  One activation row unless `rows` says otherwise.  `in_kind` selects where the activation
  * row x [K] comes from, `out_kind` what happens to the finished row o [N]; only the fields of the
  * selected kinds are read.
  *
@@ -168,7 +168,13 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
  * The sum of squares of KX_OUT_RESIDUAL / KX_IN_NORM is added tile by tile, an order of its own:
  * results agree with kx_add_rmsnorm_bf16 followed by the GEMV to within the rounding of that sum
  * (an occasional last-bit difference in the normalised row), not bit for bit.
- * Always the vector kernel.  Replaces: the chain LayerMHA -> LayerMatmul -> LayerAdd -> LayerRMSNorm ->
+ * With rows = 2 .. KX_MAX_BATCH every tensor gains a leading dimension (x [rows, K], y / residual_* [rows, N],
+ * norm_sumsq [rows, norm_parts], sumsq_out [rows, ceil(N / 256)]); gate, up and norm_row may have their rows
+ * act_ld elements apart.  That form runs on the matrix-core kernel and takes KX_IN_ROW / KX_IN_SWIGLU /
+ * KX_IN_NORM with KX_OUT_ROW / KX_OUT_RESIDUAL, a power-of-two group size, N a multiple of 16, act_ld a
+ * multiple of 8 and 16-byte aligned gate / up / norm_row / norm_gain; with SwiGLU input and residual output it
+ * is bitwise kx_swiglu_bf16, kx_gemv_awq_bf16 and kx_add_bf16 back to back.
+ * One row: always the vector kernel.  Replaces: the chain LayerMHA -> LayerMatmul -> LayerAdd -> LayerRMSNorm ->
  * LayerMatmul -> LayerSwiGLU -> LayerMatmul -> LayerAdd -> LayerRMSNorm of a decoder layer, one link
  * per call (slots kuiper/include/op/layer.h:8-20; none implemented in the reference).
  * ------------------------------------------------------------------------------------------ */
@@ -314,6 +320,31 @@ int kx_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int32_t n, 
 int kx_embedding_bf16(const uint16_t* table, const int32_t* token, uint16_t* out, int32_t vocab, int32_t dim,
                       void* stream);
 int kx_argmax_bf16(const uint16_t* x, int32_t n, int32_t* out_index, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * The same for `batch` (1 .. KX_MAX_BATCH) sequences decoded together.  Row b of every activation
+ * tensor belongs to sequence b; sequence b has its own position pos[b] and its own cache pair, which
+ * starts b * cache_stride elements into k_cache / v_cache (cache_stride a multiple of 8 and at least
+ * positions * n_kv_heads * 128).  Per sequence the arithmetic is that of the one-sequence calls, bit for bit.
+ *   kx_qk_norm_rope_batch_bf16   qkv [batch, (n_q + 2 n_kv) * 128], q_out [batch, n_q * 128]
+ *   kx_attn_decode_batch_bf16    q, out [batch, n_q * 128]; workspace of batch *
+ *                                kx_attn_decode_workspace_bytes(...) bytes
+ *   kx_embedding_rows_bf16       out[r, :] = table[tokens[r], :]
+ *   kx_argmax_rows_bf16          out_index[r] = argmax of x[r * ld .. r * ld + n - 1]
+ * The GEMVs of such a step take their rows through M (kx_gemv_awq_bf16, kx_gemv_bf16) or through
+ * kx_chain_desc.rows.  No counterpart in the reference, whose decode slots are empty (see above).
+ * ------------------------------------------------------------------------------------------ */
+int kx_qk_norm_rope_batch_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain, uint16_t* q_out,
+                               uint16_t* k_cache, uint16_t* v_cache, size_t cache_stride, int32_t n_q_heads,
+                               int32_t n_kv_heads, int32_t head_dim, const int32_t* pos, int32_t cache_positions,
+                               float rope_theta, float eps, int32_t batch, void* stream);
+int kx_attn_decode_batch_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                              size_t cache_stride, uint16_t* out, int32_t n_q_heads, int32_t n_kv_heads,
+                              int32_t head_dim, const int32_t* pos, int32_t max_positions, void* workspace,
+                              size_t workspace_bytes, int32_t batch, void* stream);
+int kx_embedding_rows_bf16(const uint16_t* table, const int32_t* tokens, uint16_t* out, int32_t vocab, int32_t dim,
+                           int32_t rows, void* stream);
+int kx_argmax_rows_bf16(const uint16_t* x, int32_t n, int32_t ld, int32_t* out_index, int32_t rows, void* stream);
 
 #ifdef __cplusplus
 }

@@ -45,6 +45,11 @@ SIGNATURES = {
     "kx_add_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _P]),
     "kx_embedding_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _P]),
     "kx_argmax_bf16": (ctypes.c_int, [_P, _I32, _P, _P]),
+    "kx_qk_norm_rope_batch_bf16": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _SZ, _I32, _I32, _I32, _P, _I32,
+                                                  ctypes.c_float, ctypes.c_float, _I32, _P]),
+    "kx_attn_decode_batch_bf16": (ctypes.c_int, [_P, _P, _P, _SZ, _P, _I32, _I32, _I32, _P, _I32, _P, _SZ, _I32, _P]),
+    "kx_embedding_rows_bf16": (ctypes.c_int, [_P, _P, _P, _I32, _I32, _I32, _P]),
+    "kx_argmax_rows_bf16": (ctypes.c_int, [_P, _I32, _I32, _P, _I32, _P]),
     "kx_awq_dequant_bf16": (ctypes.c_int, [_P, _P, _P, _P, _I32, _I32, _I32, _P]),
 }
 
@@ -326,6 +331,42 @@ def add_bf16(a, b, out):
 
 def embedding_bf16(table, token, out):
     _check(load().kx_embedding_bf16(_ptr(table), _ptr(token), _ptr(out), table.shape[0], table.shape[1], _stream()))
+
+
+def qk_norm_rope_batch_bf16(qkv, q_gain, k_gain, q_out, k_cache, v_cache, n_q, n_kv, pos, theta, eps):
+    """Batched form: qkv [B, (n_q + 2 n_kv) * 128], caches [B, positions, n_kv, 128] (any stride between
+    sequences), pos int32 [B]."""
+    B = qkv.shape[0]
+    if k_cache.stride(0) != v_cache.stride(0):
+        raise ValueError("the K and V caches must share the stride between sequences")
+    _check(load().kx_qk_norm_rope_batch_bf16(_ptr(qkv), _ptr(q_gain), _ptr(k_gain), _ptr(q_out), _ptr(k_cache),
+                                             _ptr(v_cache), k_cache.stride(0), n_q, n_kv, 128, _ptr(pos),
+                                             min(k_cache.shape[1], v_cache.shape[1]), theta, eps, B, _stream()))
+
+
+def attn_decode_batch_workspace(batch, n_q, max_positions, device="cuda"):
+    import torch
+    nbytes = int(load().kx_attn_decode_workspace_bytes(n_q, 128, max_positions))
+    return torch.empty(batch * nbytes, dtype=torch.uint8, device=device)
+
+
+def attn_decode_batch_bf16(q, k_cache, v_cache, out, n_q, n_kv, pos, max_positions, workspace):
+    B = q.shape[0]
+    if k_cache.stride(0) != v_cache.stride(0):
+        raise ValueError("the K and V caches must share the stride between sequences")
+    _check(load().kx_attn_decode_batch_bf16(_ptr(q), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), _ptr(out), n_q,
+                                            n_kv, 128, _ptr(pos), max_positions, _ptr(workspace),
+                                            workspace.numel(), B, _stream()))
+
+
+def embedding_rows_bf16(table, tokens, out):
+    _check(load().kx_embedding_rows_bf16(_ptr(table), _ptr(tokens), _ptr(out), table.shape[0], table.shape[1],
+                                         tokens.numel(), _stream()))
+
+
+def argmax_rows_bf16(x, out_index):
+    rows, n = x.shape
+    _check(load().kx_argmax_rows_bf16(_ptr(x), n, x.stride(0), _ptr(out_index), rows, _stream()))
 
 
 def argmax_bf16(x, out_index):

@@ -354,15 +354,45 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
 #endif
     if constexpr (EPI == kEpiResidual) {
         static_assert(THREADS == kTileCols, "the residual epilogue is laid out for 256 threads");
+        // Thread t ends up with the finished sums of tile column t, every row; the residual rows are
+        // requested as soon as the workgroup knows that it is the one to finish.
         float sum[ROWS];
-        if (!splitk_exchange_sum<ROWS>(psum, sum, 0, M, N, ct, kt, ktiles, ct, partials, counters, &s_prev)) return;
+        uint16_t rin[ROWS];
+        auto load_residual = [&] {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) rin[r] = res.in[static_cast<size_t>(r < M ? r : M - 1) * N + own_ld];
+        };
+        if constexpr (ROWS >= 4) {
+            // the wide read-back hands out two columns and half of the rows per thread: through LDS (the
+            // reduction buffer, free again) to one column and every row per thread
+            float* s_sum = &red[0][0][0];
+            static_assert(WAVES * MC >= ROWS, "the reduction buffer holds a tile of finished sums");
+            if (ktiles == 1) {
+                load_residual();
+#pragma unroll
+                for (int r = 0; r < ROWS; r++) sum[r] = psum[r];
+            } else {
+                constexpr int HALF = ROWS / 2;
+                float lo[HALF], hi[HALF];
+                if (!splitk_exchange_sum_wide<ROWS>(psum, lo, hi, M, N, ct, kt, ktiles, partials, counters, &s_prev,
+                                                    load_residual)) {
+                    return;
+                }
+                const int row0 = (tid / (kTileCols / 2)) * HALF;
+#pragma unroll
+                for (int i = 0; i < HALF; i++) {
+                    *reinterpret_cast<f32x2*>(&s_sum[(row0 + i) * kTileCols + 2 * (tid % (kTileCols / 2))]) = f32x2{lo[i], hi[i]};
+                }
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < ROWS; r++) sum[r] = s_sum[r * kTileCols + tid];
+            }
+        } else {
+            if (!splitk_exchange_sum<ROWS>(psum, sum, 0, M, N, ct, kt, ktiles, ct, partials, counters, &s_prev)) return;
+            load_residual();
+        }
         __shared__ float s_quarter[ROWS][kTileCols / kWave];
         const bool col_ok = own_col < N;
-        uint16_t rin[ROWS];
-#pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            rin[r] = res.in[static_cast<size_t>(r < M ? r : M - 1) * N + own_ld];
-        }
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             float rv = 0.0f;

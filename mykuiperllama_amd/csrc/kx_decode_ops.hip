@@ -109,11 +109,20 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(uint16_t* __restr
 //   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
 //   out[i + 64] = x[i+64] * cos(pos f_i) + x[i] * sin(pos f_i),     f_i = theta^(-i/64)
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __restrict__ qkv, RopeTarget t) {
+// Several sequences decoded together: blockIdx.y is the sequence; row b of qkv and q_out, position pos[b] and
+// the cache pair that starts b * cache_stride elements into k_cache / v_cache belong to sequence b.
+__global__ __launch_bounds__(256) void qk_norm_rope_kernel(const uint16_t* __restrict__ qkv, RopeTarget t,
+                                                           size_t cache_stride) {
     const int head = blockIdx.x * 4 + threadIdx.x / kWave;  // 0 .. n_q + 2 n_kv - 1
     const int lane = threadIdx.x % kWave;
-    if (head >= t.n_q + 2 * t.n_kv) return;
-    const uint16_t* src = qkv + static_cast<size_t>(head) * kHeadDim;
+    const int heads = t.n_q + 2 * t.n_kv;
+    if (head >= heads) return;
+    const size_t seq = blockIdx.y;
+    t.q_out += seq * t.n_q * kHeadDim;
+    t.k_cache += seq * cache_stride;
+    t.v_cache += seq * cache_stride;
+    t.pos += seq;
+    const uint16_t* src = qkv + (seq * heads + head) * kHeadDim;
     qk_norm_rope_head(src[lane], src[lane + 64], head, lane, t);
 }
 
@@ -135,7 +144,7 @@ template <int CHUNK>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     float* __restrict__ part_out, float* __restrict__ part_ml, int n_kv, int G, const int32_t* __restrict__ pos_ptr,
-    int nchunks, int max_positions, float scale) {
+    int nchunks, int max_positions, float scale, size_t cache_stride) {
     // Scores, then softmax weights, per head; rows padded so that the sixteen-byte reads of the
     // second pass (one row per lane) do not all start on the same bank.
     __shared__ __attribute__((aligned(16))) float s_score[kMaxGroup][CHUNK + 4];
@@ -149,6 +158,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const int chunk = blockIdx.x;
     const int p0 = chunk * CHUNK;
     const int tid = threadIdx.x;
+    {
+        // several sequences decoded together: blockIdx.z is the sequence, with its own query row, cache pair
+        // (cache_stride elements apart), position and slice of the two result arrays
+        const size_t seq = blockIdx.z;
+        const size_t heads = static_cast<size_t>(n_kv) * G;
+        q += seq * heads * kHeadDim;
+        k_cache += seq * cache_stride;
+        v_cache += seq * cache_stride;
+        pos_ptr += seq;
+        part_out += seq * nchunks * heads * kHeadDim;
+        part_ml += seq * nchunks * heads * 2;
+    }
     const int sub = tid % 16;    // which eight dims of the row
     const int slot = tid / 16;   // position slot inside the workgroup: 16 slots
 
@@ -331,6 +352,13 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
     const int kvh = head / G;
     const int g = head % G;
     const int tid = threadIdx.x;
+    {
+        const size_t seq = blockIdx.y;  // several sequences decoded together
+        const size_t heads = gridDim.x;
+        part_out += seq * nchunks * heads * kHeadDim;
+        part_ml += seq * nchunks * heads * 2;
+        out += seq * heads * kHeadDim;
+    }
     // thread (part, d) sums dimension d over the chunks c = part, part + 4, ...
     const int d = tid % kHeadDim;
     const int part = tid / kHeadDim;
@@ -423,11 +451,12 @@ __global__ __launch_bounds__(256) void add_bf16_kernel(const uint16_t* __restric
 __global__ __launch_bounds__(256) void embedding_kernel(const uint16_t* __restrict__ table,
                                                         const int32_t* __restrict__ token_ptr,
                                                         uint16_t* __restrict__ out, int chunks, int vocab) {
-    int token = token_ptr[0];
+    int token = token_ptr[blockIdx.y];  // blockIdx.y: which of the tokens looked up together
     token = token < 0 ? 0 : (token >= vocab ? vocab - 1 : token);
     const uint4* row = reinterpret_cast<const uint4*>(table + static_cast<size_t>(token) * chunks * 8);
+    uint4* dst = reinterpret_cast<uint4*>(out) + static_cast<size_t>(blockIdx.y) * chunks;
     for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += gridDim.x * blockDim.x) {
-        reinterpret_cast<uint4*>(out)[c] = row[c];
+        dst[c] = row[c];
     }
 }
 
@@ -437,7 +466,9 @@ __global__ __launch_bounds__(256) void embedding_kernel(const uint16_t* __restri
 // first index that holds it, and only in the threads whose own maximum is the overall one.
 constexpr int kArgmaxThreads = 1024;
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const uint16_t* __restrict__ x, int n,
-                                                               int32_t* __restrict__ out) {
+                                                               int32_t* __restrict__ out, size_t ld) {
+    x += blockIdx.x * ld;  // one workgroup per row
+    out += blockIdx.x;
     constexpr int kWaves = kArgmaxThreads / kWave;
     __shared__ float s_val[kWaves];
     __shared__ int s_idx[kWaves];
@@ -571,10 +602,27 @@ extern "C" int kx_qk_norm_rope_bf16(const uint16_t* qkv, const uint16_t* q_gain,
     if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || cache_positions < 1 || !(rope_theta > 1.0f)) {
         return KX_ERR_BAD_SHAPE;
     }
+    return kx_qk_norm_rope_batch_bf16(qkv, q_gain, k_gain, q_out, k_cache, v_cache, 0, n_q_heads, n_kv_heads, head_dim,
+                                      pos, cache_positions, rope_theta, eps, 1, stream);
+}
+
+extern "C" int kx_qk_norm_rope_batch_bf16(const uint16_t* qkv, const uint16_t* q_gain, const uint16_t* k_gain,
+                                          uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, size_t cache_stride,
+                                          int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos,
+                                          int32_t cache_positions, float rope_theta, float eps, int32_t batch,
+                                          void* stream) {
+    if (!qkv || !q_gain || !k_gain || !q_out || !k_cache || !v_cache || !pos) return KX_ERR_NULL_POINTER;
+    if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || cache_positions < 1 || !(rope_theta > 1.0f) ||
+        batch < 1 || batch > KX_MAX_BATCH) {
+        return KX_ERR_BAD_SHAPE;
+    }
+    // consecutive caches must not overlap
+    if (batch > 1 && cache_stride < static_cast<size_t>(cache_positions) * n_kv_heads * kx::kHeadDim) return KX_ERR_BAD_SHAPE;
     const int heads = n_q_heads + 2 * n_kv_heads;
     kx::RopeTarget t{q_gain, k_gain, q_out, k_cache, v_cache, pos, cache_positions, n_q_heads, n_kv_heads,
                      log2f(rope_theta), eps};
-    hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4), dim3(256), 0, kx::as_stream(stream), qkv, t);
+    hipLaunchKernelGGL(kx::qk_norm_rope_kernel, dim3((heads + 3) / 4, batch), dim3(256), 0, kx::as_stream(stream), qkv,
+                       t, cache_stride);
     return kx::launch_status();
 }
 
@@ -588,36 +636,41 @@ namespace {
 // Shared by the two attention entry points: checks, then the first stage and (with `out`) the merge.
 int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, uint16_t* out,
                 int32_t n_q_heads, int32_t n_kv_heads, int32_t head_dim, const int32_t* pos, int32_t max_positions,
-                void* workspace, size_t workspace_bytes, void* stream) {
+                void* workspace, size_t workspace_bytes, void* stream, int32_t batch = 1, size_t cache_stride = 0) {
     if (!q || !k_cache || !v_cache || !pos || !workspace) return KX_ERR_NULL_POINTER;
     if (head_dim != kx::kHeadDim || n_q_heads < 1 || n_kv_heads < 1 || (n_q_heads % n_kv_heads) != 0 ||
-        max_positions < 1) {
+        max_positions < 1 || batch < 1 || batch > KX_MAX_BATCH) {
         return KX_ERR_BAD_SHAPE;
     }
     const int G = n_q_heads / n_kv_heads;
     if (G > kx::kMaxGroup) return KX_ERR_BAD_SHAPE;
-    if (workspace_bytes < kx_attn_decode_workspace_bytes(n_q_heads, head_dim, max_positions)) return KX_ERR_WORKSPACE;
+    if (batch > 1 && ((cache_stride % 8) != 0 ||
+                      cache_stride < static_cast<size_t>(max_positions) * n_kv_heads * kx::kHeadDim)) {
+        return KX_ERR_BAD_SHAPE;  // every cache 16-byte aligned, none inside another
+    }
+    if (workspace_bytes < batch * kx_attn_decode_workspace_bytes(n_q_heads, head_dim, max_positions)) return KX_ERR_WORKSPACE;
     if (!kx::aligned16(q) || !kx::aligned16(k_cache) || !kx::aligned16(v_cache) || !kx::aligned16(workspace)) {
         return KX_ERR_ALIGNMENT;
     }
     const int nchunks = kx::attn_chunks_of(max_positions);
     if (nchunks > kx::kMergeLanesLong * kx::kWave) return KX_ERR_BAD_SHAPE;  // 65536 positions
     const bool long_chunks = kx::attn_chunk_for(max_positions) == kx::kAttnChunkLong;
+    // the unnormalised vectors of every sequence first, then the statistics of every sequence
     float* part_out = static_cast<float*>(workspace);
-    float* part_ml = part_out + static_cast<size_t>(nchunks) * n_q_heads * kx::kHeadDim;
+    float* part_ml = part_out + static_cast<size_t>(batch) * nchunks * n_q_heads * kx::kHeadDim;
     const float scale = 1.0f / sqrtf(static_cast<float>(kx::kHeadDim));
     hipStream_t s = kx::as_stream(stream);
-    dim3 grid1(nchunks, n_kv_heads);
+    dim3 grid1(nchunks, n_kv_heads, batch);
     if (long_chunks) {
         hipLaunchKernelGGL((kx::attn_decode_stage1<kx::kAttnChunkLong>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache,
-                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale);
+                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale, cache_stride);
     } else {
         hipLaunchKernelGGL((kx::attn_decode_stage1<kx::kAttnChunkShort>), grid1, dim3(kx::kAttnThreads), 0, s, q, k_cache,
-                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale);
+                           v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale, cache_stride);
     }
     if (out) {
-        hipLaunchKernelGGL(kx::attn_decode_stage2, dim3(n_q_heads), dim3(kx::kMergeThreads), nchunks * sizeof(float), s,
-                           part_out, part_ml, out, G, nchunks);
+        hipLaunchKernelGGL(kx::attn_decode_stage2, dim3(n_q_heads, batch), dim3(kx::kMergeThreads),
+                           nchunks * sizeof(float), s, part_out, part_ml, out, G, nchunks);
     }
     return kx::launch_status();
 }
@@ -630,6 +683,15 @@ extern "C" int kx_attn_decode_bf16(const uint16_t* q, const uint16_t* k_cache, c
     if (!out) return KX_ERR_NULL_POINTER;
     return attn_decode(q, k_cache, v_cache, out, n_q_heads, n_kv_heads, head_dim, pos, max_positions, workspace,
                        workspace_bytes, stream);
+}
+
+extern "C" int kx_attn_decode_batch_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                                         size_t cache_stride, uint16_t* out, int32_t n_q_heads, int32_t n_kv_heads,
+                                         int32_t head_dim, const int32_t* pos, int32_t max_positions, void* workspace,
+                                         size_t workspace_bytes, int32_t batch, void* stream) {
+    if (!out) return KX_ERR_NULL_POINTER;
+    return attn_decode(q, k_cache, v_cache, out, n_q_heads, n_kv_heads, head_dim, pos, max_positions, workspace,
+                       workspace_bytes, stream, batch, cache_stride);
 }
 
 extern "C" int kx_attn_decode_partial_bf16(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
@@ -667,15 +729,29 @@ extern "C" int kx_embedding_bf16(const uint16_t* table, const int32_t* token, ui
     if (!table || !token || !out) return KX_ERR_NULL_POINTER;
     if (vocab < 1 || dim < 8 || (dim % 8) != 0) return KX_ERR_BAD_SHAPE;
     if (!kx::aligned16(table) || !kx::aligned16(out)) return KX_ERR_ALIGNMENT;
+    return kx_embedding_rows_bf16(table, token, out, vocab, dim, 1, stream);
+}
+
+extern "C" int kx_embedding_rows_bf16(const uint16_t* table, const int32_t* tokens, uint16_t* out, int32_t vocab,
+                                      int32_t dim, int32_t rows, void* stream) {
+    if (!table || !tokens || !out) return KX_ERR_NULL_POINTER;
+    if (vocab < 1 || dim < 8 || (dim % 8) != 0 || rows < 1 || rows > 65535) return KX_ERR_BAD_SHAPE;
+    if (!kx::aligned16(table) || !kx::aligned16(out)) return KX_ERR_ALIGNMENT;
     const int chunks = dim / 8;
-    hipLaunchKernelGGL(kx::embedding_kernel, dim3((chunks + 255) / 256), dim3(256), 0, kx::as_stream(stream), table,
-                       token, out, chunks, vocab);
+    hipLaunchKernelGGL(kx::embedding_kernel, dim3((chunks + 255) / 256, rows), dim3(256), 0, kx::as_stream(stream),
+                       table, tokens, out, chunks, vocab);
     return kx::launch_status();
 }
 
 extern "C" int kx_argmax_bf16(const uint16_t* x, int32_t n, int32_t* out_index, void* stream) {
+    return kx_argmax_rows_bf16(x, n, n, out_index, 1, stream);
+}
+
+extern "C" int kx_argmax_rows_bf16(const uint16_t* x, int32_t n, int32_t ld, int32_t* out_index, int32_t rows,
+                                   void* stream) {
     if (!x || !out_index) return KX_ERR_NULL_POINTER;
-    if (n < 1) return KX_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(kx::argmax_kernel, dim3(1), dim3(kx::kArgmaxThreads), 0, kx::as_stream(stream), x, n, out_index);
+    if (n < 1 || rows < 1 || (rows > 1 && ld < n)) return KX_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(kx::argmax_kernel, dim3(rows), dim3(kx::kArgmaxThreads), 0, kx::as_stream(stream), x, n,
+                       out_index, static_cast<size_t>(ld));
     return kx::launch_status();
 }

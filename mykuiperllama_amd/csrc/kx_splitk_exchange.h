@@ -159,33 +159,27 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
     }
 }
 
-// The exchange with the plain epilogue for several activation rows (ROWS = 4, 8 or 16) and a workgroup of
-// exactly 256 threads.  Partial sums go out as above, one column per thread.  The last workgroup
-// reads them back two columns per load: threads 0..127 take rows 0 .. ROWS/2-1 of column pairs
-// 0..127, threads 128..255 the other rows, so a K tile costs a thread ROWS/2 eight-byte loads
-// instead of ROWS four-byte ones and every K tile of the usual shapes is in flight at once.
-// Per output the additions run t = 0, 1, 2, ... as in the narrow exchange.
-template <int ROWS>
-__device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[ROWS], int M, int N, int ct, int kt,
-                                                           int ktiles, float* __restrict__ partials,
-                                                           uint32_t* __restrict__ counters,
-                                                           uint16_t* __restrict__ y, uint32_t* s_prev) {
+// The exchange for several activation rows (ROWS = 4, 8 or 16) and a workgroup of exactly 256 threads, more
+// than one K tile.  Partial sums go out as above, one column per thread.  The last workgroup reads them back
+// two columns per load: threads 0..127 take rows 0 .. ROWS/2-1 of column pairs 0..127, threads 128..255 the
+// other rows, so a K tile costs a thread ROWS/2 eight-byte loads instead of ROWS four-byte ones and every
+// K tile of the usual shapes is in flight at once.  Per output the additions run t = 0, 1, 2, ... as in
+// the narrow exchange.
+// Returns true, the same in every thread, in the workgroup that ends up with the finished sums: thread tid
+// then holds rows (tid / 128) * ROWS/2 + i, i < ROWS/2, of columns 2 (tid % 128) (`lo`) and the next one
+// (`hi`) of the tile.  `before_read_back()` runs in that workgroup once it knows it is the last one, ahead
+// of the read-back: loads issued there return under the read-back's round trip.
+template <int ROWS, class Before>
+__device__ __forceinline__ bool splitk_exchange_sum_wide(const float (&psum)[ROWS], float (&lo)[ROWS / 2],
+                                                         float (&hi)[ROWS / 2], int M, int N, int ct, int kt,
+                                                         int ktiles, float* __restrict__ partials,
+                                                         uint32_t* __restrict__ counters, uint32_t* s_prev,
+                                                         Before&& before_read_back) {
     static_assert(ROWS == 4 || ROWS == 8 || ROWS == 16, "row counts the wide read-back is laid out for");
     const int tid = threadIdx.x;
     const int col = ct * kTileCols + tid;
-    const bool col_ok = col < N;
-    if (ktiles == 1) {
-        if (col_ok) {
-#pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                if (r < M) y[static_cast<size_t>(r) * N + col] = f32_to_bf16(psum[r]);
-            }
-        }
-        return;
-    }
-
     const size_t tstride = static_cast<size_t>(M) * N;
-    if (col_ok) {
+    if (col < N) {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             if (r < M) store_agent(partials + static_cast<size_t>(kt) * tstride + static_cast<size_t>(r) * N + col, psum[r]);
@@ -199,7 +193,8 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
         *s_prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return;
+    if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return false;
+    before_read_back();
 
     constexpr int HALF = ROWS / 2;   // rows per thread
     constexpr int TB = HALF >= 4 ? 64 / HALF : 16;  // K tiles per batch: up to 64 loads in flight
@@ -213,11 +208,10 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
         partials, 0, static_cast<int>(static_cast<uint32_t>(static_cast<size_t>(ktiles) * tstride * sizeof(float))),
         0x00020000);
     constexpr int kDeviceScope = 16;
+#pragma unroll
+    for (int i = 0; i < HALF; i++) lo[i] = hi[i] = 0.0f;
     if (col2 < static_cast<unsigned>(N)) {  // N is even: a pair is all in or all out
         const int lane_bytes = static_cast<int>(col2 * sizeof(float));
-        float lo[HALF], hi[HALF];
-#pragma unroll
-        for (int i = 0; i < HALF; i++) lo[i] = hi[i] = 0.0f;
         for (int t0 = 0; t0 < ktiles; t0 += TB) {
             // two scalars per load: a bit cast applied to one element of a vector (v.y) reads
             // element 0 with this compiler
@@ -248,6 +242,37 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
                 }
             }
         }
+    }
+    if (tid == 0) {
+        // leave the workspace ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+
+// The wide exchange followed by the plain epilogue: y[m, col] = bf16(sum), two columns per store.
+template <int ROWS>
+__device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[ROWS], int M, int N, int ct, int kt,
+                                                           int ktiles, float* __restrict__ partials,
+                                                           uint32_t* __restrict__ counters,
+                                                           uint16_t* __restrict__ y, uint32_t* s_prev) {
+    const int tid = threadIdx.x;
+    if (ktiles == 1) {
+        const int col = ct * kTileCols + tid;
+        if (col < N) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (r < M) y[static_cast<size_t>(r) * N + col] = f32_to_bf16(psum[r]);
+            }
+        }
+        return;
+    }
+    constexpr int HALF = ROWS / 2;
+    float lo[HALF], hi[HALF];
+    if (!splitk_exchange_sum_wide<ROWS>(psum, lo, hi, M, N, ct, kt, ktiles, partials, counters, s_prev, [] {})) return;
+    const int row0 = __builtin_amdgcn_readfirstlane(tid / (kTileCols / 2)) * HALF;
+    const unsigned col2 = static_cast<unsigned>(ct * kTileCols + 2 * (tid % (kTileCols / 2)));
+    if (col2 < static_cast<unsigned>(N)) {
 #pragma unroll
         for (int i = 0; i < HALF; i++) {
             const int m = row0 + i;
@@ -255,10 +280,6 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
                 *reinterpret_cast<uint32_t*>(y + static_cast<size_t>(m) * N + col2) = f32x2_to_bf16x2(lo[i], hi[i]);
             }
         }
-    }
-    if (tid == 0) {
-        // leave the workspace ready for the next launch
-        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

@@ -265,6 +265,139 @@ class DecodeModel:
         return 1 + self.cfg.layers * per_layer + 1 + (2 if with_lm_head else 0)
 
 
+class BatchDecodeModel:
+    """B sequences decoded together, one token each per step: the weights of a DecodeModel, a KV cache per
+    sequence ([B, positions, n_kv, 128] per layer) and activations of B rows.  The GEMVs run on the matrix-core
+    kernel (2 <= B <= 16 rows), rotation and attention take the sequence as a grid dimension.
+
+    fused=True   seven launches per layer: q|k|v with the RMSNorm on the way in, rotation + cache append,
+                 attention (two stages), o with the residual add on the way out, gate|up with the RMSNorm on
+                 the way in, down with SwiGLU on the way in and the residual add on the way out
+    fused=False  every operator a launch of its own (SwiGLU one per sequence)
+    The two agree to the rounding of the RMSNorm's sum of squares (added per 256 columns when fused).
+    """
+
+    def __init__(self, single, batch):
+        torch = single.torch
+        if not 2 <= batch <= 16:
+            raise ValueError("2 <= batch <= 16")
+        self.torch = torch
+        self.cfg = c = single.cfg
+        self.batch = B = batch
+        self.max_positions = single.max_positions
+        self.layers, self.embed, self.lm_head, self.final_norm = single.layers, single.embed, single.lm_head, single.final_norm
+        bf = torch.bfloat16
+        self.k_cache = [torch.zeros((B, self.max_positions, c.n_kv, c.head_dim), dtype=bf, device="cuda")
+                        for _ in range(c.layers)]
+        self.v_cache = [torch.zeros((B, self.max_positions, c.n_kv, c.head_dim), dtype=bf, device="cuda")
+                        for _ in range(c.layers)]
+
+        def buf(n):
+            return torch.zeros((B, n), dtype=bf, device="cuda")
+
+        self.x = buf(c.hidden)
+        self.h = buf(c.hidden)
+        self.qkv = buf(c.qkv_out)
+        self.q = buf(c.n_q * c.head_dim)
+        self.attn = buf(c.n_q * c.head_dim)
+        self.o = buf(c.hidden)
+        self.gu = buf(2 * c.intermediate)
+        self.act = buf(c.intermediate)
+        self.down = buf(c.hidden)
+        self.logits = buf(c.vocab)
+        self.ssq = torch.zeros((B, (c.hidden + 255) // 256), dtype=torch.float32, device="cuda")
+        self.token = torch.zeros(B, dtype=torch.int32, device="cuda")
+        self.pos = torch.zeros(B, dtype=torch.int32, device="cuda")
+        self.next_token = torch.zeros(B, dtype=torch.int32, device="cuda")
+        big_k = max(c.hidden, c.intermediate, c.n_q * c.head_dim)
+        big_n = max(c.qkv_out, 2 * c.intermediate, c.hidden)
+        self.gemv_ws = capi.make_workspace(B, big_k, big_n)
+        self.attn_ws = capi.attn_decode_batch_workspace(B, c.n_q, self.max_positions)
+
+    def prefill_cache_random(self, ctx, seed=7):
+        """Rows 0 .. ctx[b]-1 of sequence b's caches get N(0,1); `ctx` is one length or one per sequence."""
+        torch = self.torch
+        lengths = [ctx] * self.batch if isinstance(ctx, int) else list(ctx)
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        for kc, vc in zip(self.k_cache, self.v_cache):
+            for b, n in enumerate(lengths):
+                kc[b, :n] = torch.randn(kc[b, :n].shape, device="cuda", generator=gen).to(torch.bfloat16)
+                vc[b, :n] = torch.randn(vc[b, :n].shape, device="cuda", generator=gen).to(torch.bfloat16)
+
+    def set_input(self, tokens, positions):
+        torch = self.torch
+        self.token.copy_(torch.as_tensor(tokens, dtype=torch.int32))
+        self.pos.copy_(torch.as_tensor(positions, dtype=torch.int32))
+
+    def _awq(self, x, w, y):
+        capi.gemv_awq_bf16(x, w[0], w[1], w[2], y, self.cfg.group, self.gemv_ws)
+
+    def _attention(self, li, L):
+        c = self.cfg
+        capi.qk_norm_rope_batch_bf16(self.qkv, L["q_norm"], L["k_norm"], self.q, self.k_cache[li], self.v_cache[li],
+                                     c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps)
+        capi.attn_decode_batch_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
+                                    self.max_positions, self.attn_ws)
+
+    def _head(self, with_lm_head):
+        if with_lm_head:
+            capi.gemv_bf16(self.h, self.lm_head, self.logits)
+            capi.argmax_rows_bf16(self.logits, self.next_token)
+
+    def step(self, with_lm_head=True, fused=True):
+        """Enqueue one step for all sequences on torch's current stream (no synchronisation)."""
+        c, B = self.cfg, self.batch
+        H, I, g, ws = c.hidden, c.intermediate, c.group, self.gemv_ws
+        capi.embedding_rows_bf16(self.embed, self.token, self.x)
+        if not fused:
+            for li, L in enumerate(self.layers):
+                if li == 0:
+                    capi.rmsnorm_bf16(self.x, L["in_norm"], self.h, c.eps)
+                else:
+                    capi.add_rmsnorm_bf16(self.x, self.down, L["in_norm"], self.h, c.eps)
+                self._awq(self.h, L["qkv"], self.qkv)
+                self._attention(li, L)
+                self._awq(self.attn, L["o"], self.o)
+                capi.add_rmsnorm_bf16(self.x, self.o, L["post_norm"], self.h, c.eps)
+                self._awq(self.h, L["gateup"], self.gu)
+                for b in range(B):  # gate and up of a row are the two halves of one gate|up output row
+                    capi.swiglu_bf16(self.gu[b, :I], self.gu[b, I:], self.act[b])
+                self._awq(self.act, L["down"], self.down)
+            capi.add_rmsnorm_bf16(self.x, self.down, self.final_norm, self.h, c.eps)
+            return self._head(with_lm_head)
+
+        x, ssq = self.x, self.ssq
+        parts = ssq.shape[1]
+        into_residual = {"out_kind": capi.OUT_RESIDUAL, "residual_in": x, "residual_out": x, "sumsq_out": ssq, "rows": B}
+        for li, L in enumerate(self.layers):
+            qw, sc, qz = L["qkv"]
+            if li == 0:  # the embedding rows come without their sums of squares
+                capi.rmsnorm_bf16(x, L["in_norm"], self.h, c.eps)
+                self._awq(self.h, L["qkv"], self.qkv)
+            else:
+                capi.gemv_awq_chain_bf16({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": ssq, "norm_parts": parts,
+                                          "norm_gain": L["in_norm"], "norm_eps": c.eps, "out_kind": capi.OUT_ROW,
+                                          "y": self.qkv, "rows": B}, qw, sc, qz, H, c.qkv_out, g, ws)
+            self._attention(li, L)
+            qw, sc, qz = L["o"]
+            capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_ROW, x=self.attn),
+                                     qw, sc, qz, c.n_q * c.head_dim, H, g, ws)
+            qw, sc, qz = L["gateup"]
+            capi.gemv_awq_chain_bf16({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": ssq, "norm_parts": parts,
+                                      "norm_gain": L["post_norm"], "norm_eps": c.eps, "out_kind": capi.OUT_ROW,
+                                      "y": self.gu, "rows": B}, qw, sc, qz, H, 2 * I, g, ws)
+            qw, sc, qz = L["down"]
+            capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_SWIGLU, gate=self.gu[:, :I], up=self.gu[:, I:],
+                                          act_ld=2 * I), qw, sc, qz, I, H, g, ws)
+        capi.rmsnorm_bf16(x, self.final_norm, self.h, c.eps)
+        return self._head(with_lm_head)
+
+    def launches_per_step(self, with_lm_head=True, fused=True):
+        per_layer = 7 if fused else 10 + self.batch
+        return 1 + self.cfg.layers * per_layer + (1 if fused else 0) + 1 + (2 if with_lm_head else 0)
+
+
 def step_bytes(cfg, ctx, with_lm_head=True):
     """Algorithmic HBM bytes of one decode step: packed projections + KV read (+ bf16 lm_head)."""
     from .synth import awq_gemv_bytes
