@@ -24,7 +24,10 @@ Prints one JSON line:  value = algorithmic bytes of a step / time of a step, in 
                 wide-load kernel through LDS), microseconds per launch
   small_batch   configs[2]: M in {1, 2, 4, 8, 16} on three shapes, microseconds per launch of the
                 vector-ALU kernel and of the MFMA kernel (cold weights, same event timing)
-  decode        configs[3] and configs[4]: tokens/s of a full decode step (Qwen3-8B, Qwen3-32B-shaped)
+  decode        configs[3] and configs[4]: tokens/s of a full decode step (Qwen3-8B, Qwen3-32B-shaped); under the
+                8B entry, small_batch_decode: 2, 8 and 16 sequences decoded together (--decode-batches), each at
+                the same position of its own KV cache, tokens/s summed over the sequences, with the GEMVs'
+                prologues and epilogues (seven launches per layer) and from stand-alone operators
 """
 import argparse
 import json
@@ -61,6 +64,8 @@ def parse_args():
     ap.add_argument("--no-decode-32b", action="store_true", help="skip the Qwen3-32B-shaped decode step")
     ap.add_argument("--decode-32b", action="store_true", help="kept for older command lines: the step runs by default")
     ap.add_argument("--decode-steps", type=int, default=60)
+    ap.add_argument("--decode-batches", default="2,8,16",
+                    help="numbers of sequences decoded together in the small_batch_decode leg (Qwen3-8B); '' skips it")
     ap.add_argument("--lib", default=None,
                     help="time another build of the HIP library (e.g. lib/libkx_hip_ablate1.so from "
                          "`python -m mykuiperllama_amd.build --ablate 1`); its numbers attribute time, its results "
@@ -488,7 +493,8 @@ def main():
     if not args.no_decode and not profiling_build:
         del sets
         torch.cuda.empty_cache()
-        d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager, batches=(2, 8, 16))
+        d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager,
+                              batches=tuple(int(b) for b in args.decode_batches.split(",") if b.strip()))
         out["decode_tok_s"] = d8["with_lm_head"]["tokens_per_s"]
         out["decode"] = {"qwen3-8b ctx4096": d8}
         if not args.no_decode_32b:

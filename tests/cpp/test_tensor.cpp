@@ -220,6 +220,21 @@ TEST_CPU(test_tensor, init_buffer_rules) {
     ASSERT_FATAL(blank.ptr<float>(0));
 }
 
+// Element counts and byte sizes are computed in size_t: the reference multiplies the int32 extents in
+// int (kuiper/source/tensor/tensor.cpp:28, :38, :49, and :57 through reduce_dims with an int seed, :6-13),
+// which wraps from 2^31 elements on.  Shape arithmetic only: the tensors borrow a pointer that is never read.
+TEST_CPU(test_tensor, element_counts_past_two_to_the_31_do_not_wrap) {
+    static char anchor;
+    tensor::Tensor table(DataType::DataTypeBf16, 151936, 16384, false, nullptr, &anchor);
+    ASSERT_EQ(table.size(), size_t(151936) * 16384);
+    ASSERT_EQ(table.byte_size(), size_t(151936) * 16384 * 2);
+    ASSERT_EQ(table.strides(), std::vector<size_t>({16384, 1}));
+    tensor::Tensor big(DataType::DataTypeFp32, std::vector<int32_t>{65536, 65536, 2}, false, nullptr, &anchor);
+    ASSERT_EQ(big.size(), size_t(1) << 33);
+    ASSERT_EQ(big.byte_size(), size_t(1) << 35);
+    ASSERT_EQ(big.strides(), std::vector<size_t>({size_t(65536) * 2, 2, 1}));
+}
+
 TEST_CPU(test_tensor, reshape_reset_index_and_new_element_types) {
     auto allocator = CPUDeviceAllocatorFactory::get_instance();
     tensor::Tensor t(DataType::DataTypeFp32, 4, 4, true, allocator);
