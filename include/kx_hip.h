@@ -102,13 +102,16 @@ int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight, const uin
 
 /* ------------------------------------------------------------------------------------------
  * The same GEMV with the activations produced on the way in, for the decode step (one launch
- * instead of two; built for M = 1, correct for M <= KX_MAX_BATCH, always the vector kernel).
- * Rounding points are those of the stand-alone kernels further down, so each call returns what
- * the two separate calls return (bitwise for kx_gemv_awq_swiglu_bf16 against the vector kernel).
+ * instead of two; M <= KX_MAX_BATCH).  Rounding points are those of the stand-alone kernels further
+ * down, so each call returns what the two separate calls return.
  *
  *   kx_gemv_awq_swiglu_bf16:  x[m,k] = bf16( bf16(silu(gate[m,k])) * up[m,k] ),  y = x W
  *       gate, up bf16, rows act_ld elements apart (act_ld >= K; halves of one [M, 2K] tensor or two
- *       tensors), 2-byte aligned.
+ *       tensors), 2-byte aligned.  Bitwise kx_swiglu_bf16 followed by kx_gemv_awq_bf16 on the same kernel:
+ *       the vector kernel at M = 1, and at M >= 2 the matrix-core kernel, as kx_gemv_awq_bf16 chooses it,
+ *       provided gate and up are 16-byte aligned and act_ld is a multiple of 8 (otherwise M >= 2 stays on
+ *       the vector kernel, two rows per workgroup).
+ *   kx_gemv_awq_addnorm_bf16 runs on the vector kernel for every M (built for M = 1).
  *   kx_gemv_awq_addnorm_bf16: r = bf16(residual + delta)   (delta may be null: r = residual)
  *                             x = gain * bf16(r * rsqrt(mean_k(r^2) + eps)),  y = x W
  *       residual, delta bf16 [M,K] (16-byte aligned), gain bf16 [K]; r is written to residual_out
