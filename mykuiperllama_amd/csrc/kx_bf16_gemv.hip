@@ -100,40 +100,55 @@ __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
 // v_mfma_f32_16x16x32_bf16 with A = the activations (row m = lane % 16, zero rows past M) and
 // B = sixteen rows of W (column n = lane % 16): lane (c, b) supplies x[c][32 s + 8 b .. + 7] and
 // W[n0 + c][32 s + 8 b .. + 7], sixteen contiguous bytes each, and receives y[4 b + v][n0 + c].
-// A workgroup owns sixteen output columns; its four waves take the 32-element steps of K in turn
-// (step s goes to wave s % 4) in sweeps of kMfmaUnroll steps with all loads of a sweep in flight
-// together, and meet in LDS.  Addresses are clamped, what lies past K or M is zeroed in both operands.
+// A workgroup owns BLOCKS blocks of sixteen output columns, which share every A operand.  One block
+// with eight steps in flight serves up to eight rows (lm_head 151936 x 4096: 270 us at M = 3..5, 300 at
+// 8); from nine rows on four blocks with four steps in flight each, so that the activation rows come out
+// of L2 once per 64 columns instead of once per 16 - at sixteen rows they are as many bytes as the sixteen
+// rows of W they meet, and with one block the L2 traffic for x equalled the HBM traffic for W (370 us at
+// M = 16, 299 with four blocks; at M = 3 four blocks are the slower choice, 297 us).  Its four waves take the
+// 32-element steps of K in turn (step s goes to wave s % 4; runs of consecutive steps per wave measured
+// slower) in sweeps of UNROLL steps with all loads of a sweep in flight together, and meet in LDS.  Addresses are clamped, what lies past K or M is zeroed
+// in both operands; per output the additions run in the same order whatever kMfmaBlocks is.
 constexpr int kMfmaWaves = 4;
-constexpr int kMfmaUnroll = 8;
 
+template <int kMfmaBlocks, int kMfmaUnroll>
 __global__ __launch_bounds__(kMfmaWaves * kWave) void bf16_gemv_mfma_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y, int M, int K, int N) {
-    __shared__ float red[kMfmaWaves][4][kWave];
+    __shared__ float red[kMfmaWaves][kMfmaBlocks][4][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int c = lane % 16;
     const int b = lane / 16;
-    const int n0 = blockIdx.x * 16;
-    const int n_ld = n0 + c < N ? n0 + c : N - 1;
+    const int n0 = blockIdx.x * 16 * kMfmaBlocks;
     const int m_ld = c < M ? c : M - 1;
-    const uint16_t* wrow = w + static_cast<size_t>(n_ld) * K;
+    const uint16_t* wrow[kMfmaBlocks];
+#pragma unroll
+    for (int j = 0; j < kMfmaBlocks; j++) {
+        const int n = n0 + 16 * j + c;
+        wrow[j] = w + static_cast<size_t>(n < N ? n : N - 1) * K;
+    }
     const uint16_t* xrow = x + static_cast<size_t>(m_ld) * K;
     const bool row_live = c < M;
     const int k_last = K - 8;  // K is a multiple of eight
 
-    f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4v acc[kMfmaBlocks];
+#pragma unroll
+    for (int j = 0; j < kMfmaBlocks; j++) acc[j] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
     constexpr int kSweep = 32 * kMfmaWaves * kMfmaUnroll;  // elements of K a workgroup covers per sweep
     for (int k0 = 32 * wave; k0 < K; k0 += kSweep) {
-        u32x4 wv[kMfmaUnroll], xv[kMfmaUnroll];
-#pragma unroll
-        for (int u = 0; u < kMfmaUnroll; u++) {
-            const int k = k0 + 32 * kMfmaWaves * u + 8 * b;
-            wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (k < K ? k : k_last)));
-        }
+        u32x4 wv[kMfmaUnroll][kMfmaBlocks], xv[kMfmaUnroll];
 #pragma unroll
         for (int u = 0; u < kMfmaUnroll; u++) {
             const int k = k0 + 32 * kMfmaWaves * u + 8 * b;
             xv[u] = *reinterpret_cast<const u32x4*>(xrow + (k < K ? k : k_last));
+        }
+#pragma unroll
+        for (int u = 0; u < kMfmaUnroll; u++) {
+            const int k = k0 + 32 * kMfmaWaves * u + 8 * b;
+#pragma unroll
+            for (int j = 0; j < kMfmaBlocks; j++) {
+                wv[u][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[j] + (k < K ? k : k_last)));
+            }
         }
         __builtin_amdgcn_sched_barrier(0);  // every load of the sweep is out before the first is waited for
 #pragma unroll
@@ -142,20 +157,29 @@ __global__ __launch_bounds__(kMfmaWaves * kWave) void bf16_gemv_mfma_kernel(
             const bool a_live = live && row_live;
             const bf16x8 a_op = as_bf16x8(a_live ? xv[u].x : 0u, a_live ? xv[u].y : 0u, a_live ? xv[u].z : 0u,
                                           a_live ? xv[u].w : 0u);
-            const bf16x8 b_op = as_bf16x8(live ? wv[u].x : 0u, live ? wv[u].y : 0u, live ? wv[u].z : 0u,
-                                          live ? wv[u].w : 0u);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, b_op, acc, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < kMfmaBlocks; j++) {
+                const bf16x8 b_op = as_bf16x8(live ? wv[u][j].x : 0u, live ? wv[u][j].y : 0u, live ? wv[u][j].z : 0u,
+                                              live ? wv[u][j].w : 0u);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, b_op, acc[j], 0, 0, 0);
+            }
         }
     }
 #pragma unroll
-    for (int v = 0; v < 4; v++) red[wave][v][lane] = acc[v];
+    for (int j = 0; j < kMfmaBlocks; j++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) red[wave][j][v][lane] = acc[j][v];
+    }
     __syncthreads();
-    if (wave == 0 && n0 + c < N) {
+    // wave j finishes block j
+    static_assert(kMfmaBlocks <= kMfmaWaves, "one wave per block of sixteen columns in the final sum");
+    const int n = n0 + 16 * wave + c;
+    if (wave < kMfmaBlocks && n < N) {
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int m = 4 * b + v;
-            const float sum = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
-            if (m < M) y[static_cast<size_t>(m) * N + n0 + c] = f32_to_bf16(sum);
+            const float sum = (red[0][wave][v][lane] + red[1][wave][v][lane]) + (red[2][wave][v][lane] + red[3][wave][v][lane]);
+            if (m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16(sum);
         }
     }
 }
@@ -175,11 +199,15 @@ extern "C" int kx_gemv_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, i
     }
     hipStream_t s = kx::as_stream(stream);
     if (M >= 3) {
-        // One pass on the matrix cores (lm_head 151936 x 4096: 270 us at M = 3..5, 300 at 8, 370 at 16;
-        // the vector kernel, whose every wave reads the activation rows for itself, needs 310 us
-        // for four rows and would need a pass over W per four rows beyond that).
-        hipLaunchKernelGGL(kx::bf16_gemv_mfma_kernel, dim3((N + 15) / 16), dim3(kx::kMfmaWaves * kx::kWave), 0, s, x, w,
-                           y, M, K, N);
+        // One pass on the matrix cores; the vector kernel, whose every wave reads the activation rows for
+        // itself, needs 310 us on lm_head 151936 x 4096 for four rows and a pass over W per four rows beyond that.
+        if (M <= 8) {
+            hipLaunchKernelGGL((kx::bf16_gemv_mfma_kernel<1, 8>), dim3((N + 15) / 16), dim3(kx::kMfmaWaves * kx::kWave), 0,
+                               s, x, w, y, M, K, N);
+        } else {
+            hipLaunchKernelGGL((kx::bf16_gemv_mfma_kernel<4, 4>), dim3((N + 63) / 64), dim3(kx::kMfmaWaves * kx::kWave), 0,
+                               s, x, w, y, M, K, N);
+        }
         return kx::launch_status();
     }
     const dim3 grid((N + kx::kRowsPerBlock - 1) / kx::kRowsPerBlock);
