@@ -139,9 +139,12 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     if constexpr (EPI == kEpiQkRope) {
         // what the wave that finishes head 2 ct + (tid / 128) will need, see the epilogue below
         const int head = ct * (kTileCols / kHeadDim) + ((tid % kTileCols) >> 7);
-        const uint16_t* gain = head < rope.n_q ? rope.q_gain : rope.k_gain;
-        rope_gain_a = gain[tid % kWave];
-        rope_gain_b = gain[tid % kWave + 64];
+        // both gains, then a select of values: a select between pointers ends up as a table in private memory
+        const bool q_head = head < rope.n_q;
+        const uint16_t qa = rope.q_gain[tid % kWave], qb = rope.q_gain[tid % kWave + 64];
+        const uint16_t ka = rope.k_gain[tid % kWave], kb = rope.k_gain[tid % kWave + 64];
+        rope_gain_a = q_head ? qa : ka;
+        rope_gain_b = q_head ? qb : kb;
         rope_pos = rope.pos[0];
     }
     float tile_ss = 0.0f;

@@ -26,6 +26,25 @@ struct RopeTarget {
     float eps;
 };
 
+// sin and cos of a rotary angle, 0 <= x < 2^17 (positions below 65536 times a frequency of at most 1).
+// The library routine carries a large-argument path that keeps a table in private memory, which makes
+// every kernel that calls it a kernel with scratch memory; the angles here never need it.  Reduction to
+// [-pi/4, pi/4] in double (x - k pi/2 with k = rint(x 2/pi): two operations, exact enough for any k below
+// 2^17), then the classic single-precision minimax polynomials (error below 1 ulp of the result) and the
+// quadrant.
+__device__ __forceinline__ void rope_sincos(float x, float* s_out, float* c_out) {
+    const float kf = rintf(x * 0.63661977236758134f);
+    const float r = static_cast<float>(__builtin_fma(static_cast<double>(-kf), 1.5707963267948966, static_cast<double>(x)));
+    const float z = r * r;
+    const float sp = r + r * z * (-1.6666654611e-1f + z * (8.3321608736e-3f + z * -1.9515295891e-4f));
+    const float cp = 1.0f - 0.5f * z + z * z * (4.166664568298827e-2f + z * (-1.388731625493765e-3f + z * 2.443315711809948e-5f));
+    const int q = static_cast<int>(kf) & 3;
+    const float sa = (q & 1) ? cp : sp;
+    const float ca = (q & 1) ? sp : cp;
+    *s_out = (q & 2) ? -sa : sa;
+    *c_out = ((q + 1) & 2) ? -ca : ca;
+}
+
 // Called by the 64 lanes of one wave; lane i brings elements i and i + 64 of head `head`
 // (0 .. n_q + 2 n_kv - 1, query heads first, then key heads, then value heads) as bf16 bits.
 //   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
@@ -58,12 +77,16 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     const float xb = bf16_to_f32(f32_to_bf16(nb));
     const float freq = exp2f(-t.log2_theta * static_cast<float>(lane) / 64.0f);
     float s, c;
-    sincosf(static_cast<float>(pos) * freq, &s, &c);
+    rope_sincos(static_cast<float>(pos) * freq, &s, &c);
     const float oa = xa * c - xb * s;
     const float ob = xb * c + xa * s;
-    uint16_t* dst = is_q ? t.q_out + static_cast<size_t>(head) * kHeadDim
-                         : t.k_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q)) * kHeadDim;
-    if (is_q || row_ok) {
+    // two guarded stores rather than one store through a selected pointer (see qk_norm_rope_head)
+    if (is_q) {
+        uint16_t* dst = t.q_out + static_cast<size_t>(head) * kHeadDim;
+        dst[lane] = f32_to_bf16(oa);
+        dst[lane + 64] = f32_to_bf16(ob);
+    } else if (row_ok) {
+        uint16_t* dst = t.k_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q)) * kHeadDim;
         dst[lane] = f32_to_bf16(oa);
         dst[lane + 64] = f32_to_bf16(ob);
     }
@@ -72,8 +95,12 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
 // The same with the three operands loaded here.
 __device__ __forceinline__ void qk_norm_rope_head(uint16_t a_bits, uint16_t b_bits, int head, int lane,
                                                   const RopeTarget& t) {
-    const uint16_t* gain = head < t.n_q ? t.q_gain : t.k_gain;  // a value head reads k_gain and ignores it
-    qk_norm_rope_head_with(a_bits, b_bits, head, lane, t, t.pos[0], gain[lane], gain[lane + 64]);
+    // both gains are read and the values selected: a select between the two pointers is compiled to a table
+    // of pointers in private memory, and a kernel with private memory is slower to start its waves
+    const bool is_q = head < t.n_q;  // a value head takes k_gain and ignores it
+    const uint16_t qa = t.q_gain[lane], qb = t.q_gain[lane + 64];
+    const uint16_t ka = t.k_gain[lane], kb = t.k_gain[lane + 64];
+    qk_norm_rope_head_with(a_bits, b_bits, head, lane, t, t.pos[0], is_q ? qa : ka, is_q ? qb : kb);
 }
 
 }  // namespace kx
