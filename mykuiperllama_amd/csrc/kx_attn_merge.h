@@ -55,10 +55,18 @@ __device__ __forceinline__ MergeStats<PER_LANE> attn_merge_load(const float* __r
     return st;
 }
 
-// Writes the factor of every chunk to s_factor[0 .. nchunks) and returns the normaliser, the same
-// value in every lane.  The result does not depend on PER_LANE (absent chunks are neutral).
+// Where the factor of chunk c lies in a table of `per_part` entries for each of the kMergeParts chunk
+// subsets: a thread that sums the chunks c = p, p + 4, ... finds its factors side by side.
+__device__ __forceinline__ int attn_factor_slot(int c, int per_part) {
+    return (c % kMergeParts) * per_part + c / kMergeParts;
+}
+
+// Writes the factor of every chunk below kMergeParts * per_part to its slot of s_factor (0 for a chunk
+// past nchunks or without a valid position, so that the sums over the table need no test on the chunk
+// count) and returns the normaliser, the same value in every lane.  The result does not depend on
+// PER_LANE (absent chunks are neutral).
 template <int PER_LANE>
-__device__ __forceinline__ float attn_merge_finish(const MergeStats<PER_LANE>& st, int nchunks, float* s_factor,
+__device__ __forceinline__ float attn_merge_finish(const MergeStats<PER_LANE>& st, float* s_factor, int per_part,
                                                    int lane) {
     float m = -INFINITY;
 #pragma unroll
@@ -69,7 +77,7 @@ __device__ __forceinline__ float attn_merge_finish(const MergeStats<PER_LANE>& s
     for (int u = 0; u < PER_LANE; u++) {
         const int c = lane + u * kWave;
         const float f = st.l[u] > 0.0f ? expf(st.m[u] - m) : 0.0f;  // chunks past the context have l == 0
-        if (c < nchunks) s_factor[c] = f;
+        if (c < kMergeParts * per_part) s_factor[attn_factor_slot(c, per_part)] = f;
         l += st.l[u] * f;
     }
     return wave_sum(l);

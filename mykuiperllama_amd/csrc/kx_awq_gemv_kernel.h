@@ -111,7 +111,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     __shared__ __attribute__((aligned(16))) float red[WAVES][kTileCols];
     __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? MB : 1][STAGED ? KB : 8];  // staged activations, bf16
     __shared__ float s_ss[NORM ? MB : 1][WAVES];
-    __shared__ float s_factor[MERGE ? HB : 1][MERGE ? kMergeParts * kMergeHold : 1];
+    __shared__ __attribute__((aligned(16))) float s_factor[MERGE ? HB : 1][MERGE ? kMergeParts * kMergeHold : 4];
     __shared__ float s_norm[MERGE ? HB : 1];
     __shared__ float s_mpart[MERGE ? kMergeParts : 1][MERGE ? KB : 1];
 
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     if constexpr (MERGE) {
         const int wave_id = tid / kWave;
         if (wave_id < HB) {
-            const float l = attn_merge_finish<kMergeStatsPerLane>(stats, fi.nchunks, s_factor[wave_id], tid % kWave);
+            const float l = attn_merge_finish<kMergeStatsPerLane>(stats, s_factor[wave_id], kMergeHold, tid % kWave);
             if (tid % kWave == 0) s_norm[wave_id] = l;
         }
         lds_barrier();
@@ -291,13 +291,23 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             const int e = tid + i * THREADS;
             const int part = e / KB;
             const int row = e % KB;
-            const float* f = s_factor[row / kHeadDim];
+            // The thread's kMergeHold factors lie side by side and chunks that do not exist carry factor 0, so
+            // the sum is straight-line code: a test on the chunk count per step had been compiled to a branch
+            // and an LDS read with a full wait per chunk, forty dependent LDS round trips per thread.
+            static_assert(kMergeHold % 4 == 0, "the factors are read four at a time");
+            const f32x4* f4 = reinterpret_cast<const f32x4*>(&s_factor[row / kHeadDim][part * kMergeHold]);
+            float f[kMergeHold];
+#pragma unroll
+            for (int j4 = 0; j4 < kMergeHold / 4; j4++) {
+                const f32x4 v = f4[j4];
+                f[4 * j4] = v.x;
+                f[4 * j4 + 1] = v.y;
+                f[4 * j4 + 2] = v.z;
+                f[4 * j4 + 3] = v.w;
+            }
             float acc_m = 0.0f;
 #pragma unroll
-            for (int j = 0; j < kMergeHold; j++) {
-                const int c = part + j * kMergeParts;
-                if (c < fi.nchunks) acc_m = attn_merge_step(acc_m, held[i][j], f[c]);
-            }
+            for (int j = 0; j < kMergeHold; j++) acc_m = attn_merge_step(acc_m, held[i][j], f[j]);
             s_mpart[part][row] = acc_m;
         }
         lds_barrier();

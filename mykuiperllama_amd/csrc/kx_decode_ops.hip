@@ -344,8 +344,11 @@ constexpr int kMergeThreads = kHeadDim * kMergeParts;
 
 __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float* __restrict__ part_out,
                                                                     const float* __restrict__ part_ml,
-                                                                    uint16_t* __restrict__ out, int G, int nchunks) {
-    extern __shared__ float s_factor[];  // nchunks rescaling factors exp(m_c - m)
+                                                                    uint16_t* __restrict__ out, int G, int nchunks,
+                                                                    int per_part) {
+    // rescaling factors exp(m_c - m), per_part slots for each of the four chunk subsets (attn_factor_slot);
+    // slots of chunks that do not exist hold 0
+    extern __shared__ __attribute__((aligned(16))) float s_factor[];
     __shared__ float s_norm;
     __shared__ float s_part[kMergeParts][kHeadDim];
     const int head = blockIdx.x;  // query head
@@ -379,16 +382,23 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
     if (tid < kWave) {
         const MergeStats<kMergeLanesLong> st =
             attn_merge_load<kMergeLanesLong>(part_ml + static_cast<size_t>(kvh) * nchunks * G * 2, g, G, nchunks, tid);
-        const float l = attn_merge_finish<kMergeLanesLong>(st, nchunks, s_factor, tid);
+        const float l = attn_merge_finish<kMergeLanesLong>(st, s_factor, per_part, tid);
         if (tid == 0) s_norm = l;
     }
     __syncthreads();
 
+    // The thread's factors lie side by side and absent chunks carry factor 0: straight-line code.  (A test
+    // on the chunk count per step had been compiled to a branch and an LDS read with a full wait per chunk.)
     float acc = 0.0f;
+    const float* fpart = s_factor + part * per_part;  // per_part >= kMergeFront, a multiple of four
+    static_assert(kMergeFront % 4 == 0, "the factors are read four at a time");
 #pragma unroll
-    for (int u = 0; u < kMergeFront; u++) {
-        const int c = part + u * kMergeParts;
-        if (c < nchunks) acc = attn_merge_step(acc, front[u], s_factor[c]);
+    for (int u4 = 0; u4 < kMergeFront / 4; u4++) {
+        const float4 f = reinterpret_cast<const float4*>(fpart)[u4];
+        acc = attn_merge_step(acc, front[4 * u4], f.x);
+        acc = attn_merge_step(acc, front[4 * u4 + 1], f.y);
+        acc = attn_merge_step(acc, front[4 * u4 + 2], f.z);
+        acc = attn_merge_step(acc, front[4 * u4 + 3], f.w);
     }
     // what a longer context leaves, in batches as before; the order of the additions is unchanged
     for (int c0 = part + kMergeFront * kMergeParts; c0 < nchunks; c0 += kMergeBatch * kMergeParts) {
@@ -403,7 +413,7 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_stage2(const float*
 #pragma unroll
         for (int u = 0; u < kMergeBatch; u++) {
             const int c = c0 + u * kMergeParts;
-            if (c < nchunks) acc = attn_merge_step(acc, v[u], s_factor[c]);
+            if (c < nchunks) acc = attn_merge_step(acc, v[u], s_factor[attn_factor_slot(c, per_part)]);
         }
     }
     s_part[part][d] = acc;
@@ -669,8 +679,12 @@ int attn_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_ca
                            v_cache, part_out, part_ml, n_kv_heads, G, pos, nchunks, max_positions, scale, cache_stride);
     }
     if (out) {
+        // slots per chunk subset: the straight-line first flight of the merge covers 32, longer contexts more
+        int per_part = (nchunks + kx::kMergeParts - 1) / kx::kMergeParts;
+        if (per_part < 32) per_part = 32;
+        per_part = (per_part + 3) / 4 * 4;
         hipLaunchKernelGGL(kx::attn_decode_stage2, dim3(n_q_heads, batch), dim3(kx::kMergeThreads),
-                           nchunks * sizeof(float), s, part_out, part_ml, out, G, nchunks);
+                           kx::kMergeParts * per_part * sizeof(float), s, part_out, part_ml, out, G, nchunks, per_part);
     }
     return kx::launch_status();
 }
