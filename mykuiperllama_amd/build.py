@@ -5,6 +5,7 @@
   test_kuiper    C++ test runner for the host API (tests/cpp/*, links oracle/kx_oracle.c)
   kx_safetensors_dump   lists the tensors of a checkpoint file (kuiper/app/safetensors_dump.cpp)
   libkx_probe.so  measurement only: the streaming-read kernel bench.py uses as the floor (probe/*.hip)
+  test_kuiper_asan  optional (--asan): the host API and its C++ tests with AddressSanitizer on the host code
 
 `python -m mykuiperllama_amd.build --ablate N` additionally builds lib/libkx_hip_ablateN.so, the HIP
 library with parts of the GEMV kernels compiled out (-DKX_ABLATE=N: 1 = no split-K exchange, 2 = loads
@@ -93,6 +94,34 @@ def build_kuiper():
     return KUIPER_LIB
 
 
+def build_kuiper_asan():
+    """The C++ host API and its tests as one binary with AddressSanitizer on the host code (the device code
+    is compiled as usual): lib/test_kuiper_asan.  Run it with ASAN_OPTIONS=protect_shadow_gap=0 (the HIP
+    runtime maps memory where the sanitizer keeps a gap); at process exit the sanitizer's own allocator may
+    trip over the already unloaded HIP runtime, after the tests have reported."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(LIB_DIR, "obj_asan")
+    os.makedirs(obj_dir, exist_ok=True)
+    inc = ["-I", INCLUDE, "-I", os.path.join(KUIPER, "include"), "-I", os.path.join(KUIPER, "source", "op"),
+           "-I", TESTS_CPP]
+    asan = ["-O1", "-g", "-std=c++17", "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fno-omit-frame-pointer"]
+    srcs = sorted(glob.glob(os.path.join(KUIPER, "source", "**", "*.cpp"), recursive=True) +
+                  glob.glob(os.path.join(KUIPER, "source", "**", "*.hip"), recursive=True) +
+                  glob.glob(os.path.join(TESTS_CPP, "*.cpp")) + glob.glob(os.path.join(TESTS_CPP, "*.hip")))
+    oracle_obj = os.path.join(obj_dir, "kx_oracle.o")
+    _run(["gcc", "-O1", "-g", "-fPIC", "-std=c11", "-fsanitize=address", "-c",
+          os.path.join(ROOT, "oracle", "kx_oracle.c"), "-o", oracle_obj])
+    objs = [oracle_obj]
+    for i, src in enumerate(srcs):
+        obj = os.path.join(obj_dir, f"{i}_{os.path.basename(src)}.o")
+        _run([HIPCC] + DEVICE_FLAGS + asan + inc + ["-c", src, "-o", obj])
+        objs.append(obj)
+    out = os.path.join(LIB_DIR, "test_kuiper_asan")
+    _run([HIPCC, "--offload-arch=gfx950", "-fsanitize=address"] + objs +
+         ["-L", LIB_DIR, "-lkx_hip", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
+
+
 def build_all():
     build_kx()
     build_kuiper()
@@ -103,8 +132,11 @@ if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser()
     ap.add_argument("--ablate", type=int, default=0, help="also build lib/libkx_hip_ablateN.so (profiling only)")
+    ap.add_argument("--asan", action="store_true", help="also build lib/test_kuiper_asan (host code under AddressSanitizer)")
     args = ap.parse_args()
     build_all()
     print("built:", KX_LIB, KUIPER_LIB if os.path.exists(KUIPER_LIB) else "", PROBE_LIB)
     if args.ablate:
         print("built:", build_kx(args.ablate))
+    if args.asan:
+        print("built:", build_kuiper_asan())
