@@ -174,7 +174,8 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
  * With rows = 2 .. KX_MAX_BATCH every tensor gains a leading dimension (x [rows, K], y / residual_* [rows, N],
  * norm_sumsq [rows, norm_parts], sumsq_out [rows, ceil(N / 256)]); gate, up and norm_row may have their rows
  * act_ld elements apart.  That form runs on the matrix-core kernel and takes KX_IN_ROW / KX_IN_SWIGLU /
- * KX_IN_NORM with KX_OUT_ROW / KX_OUT_RESIDUAL, a power-of-two group size, N a multiple of 16, act_ld a
+ * KX_IN_NORM with any output kind (KX_OUT_QKV_ROPE: q_out [rows, n_q * 128], pos [rows], one cache pair per
+ * row, see cache_stride), a power-of-two group size, N a multiple of 16, act_ld a
  * multiple of 8 and 16-byte aligned gate / up / norm_row / norm_gain; with SwiGLU input and residual output it
  * is bitwise kx_swiglu_bf16, kx_gemv_awq_bf16 and kx_add_bf16 back to back.
  * One row: always the vector kernel.  Replaces: the chain LayerMHA -> LayerMatmul -> LayerAdd -> LayerRMSNorm ->
@@ -232,6 +233,9 @@ typedef struct kx_chain_desc {
      * consecutive rows of gate / up / norm_row (0 reads as K) */
     int32_t rows;
     int32_t act_ld;
+    /* KX_OUT_QKV_ROPE with rows > 1: row m is sequence m, with position pos[m] and the cache pair that
+     * starts m * cache_stride elements into k_cache / v_cache (at least cache_positions * n_kv_heads * 128) */
+    size_t cache_stride;
 } kx_chain_desc;
 
 int kx_gemv_awq_chain_bf16(const kx_chain_desc* desc, const int32_t* qweight, const uint16_t* scales,

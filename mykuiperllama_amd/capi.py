@@ -74,7 +74,7 @@ class ChainDesc(ctypes.Structure):
         ("y", _P),
         ("residual_in", _P), ("residual_out", _P), ("sumsq_out", _P),
         ("q_gain", _P), ("k_gain", _P), ("q_out", _P), ("k_cache", _P), ("v_cache", _P), ("pos", _P),
-        ("rows", _I32), ("act_ld", _I32),
+        ("rows", _I32), ("act_ld", _I32), ("cache_stride", _SZ),
     ]
 
 

@@ -256,10 +256,11 @@ void launch_fused(const AwqPlan& p, const FusedInput& fi, const int32_t* qweight
 template <int PRO, int EPI>
 void launch_mfma_fused(const AwqPlan& p, const FusedInput& fi, const ResidualTarget& res, const uint16_t* x,
                        const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros, uint16_t* y,
-                       float* partials, uint32_t* counters, int M, int K, int N, int group, hipStream_t stream) {
+                       float* partials, uint32_t* counters, int M, int K, int N, int group, hipStream_t stream,
+                       const RopeTarget& rope = RopeTarget{}, size_t cache_stride = 0) {
     int group_shift = 0;
     while ((1 << group_shift) < group) group_shift++;
-#define KX_MARGS x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_shift, p.coltiles, p.ktiles, stream, fi, res
+#define KX_MARGS x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_shift, p.coltiles, p.ktiles, stream, fi, res, rope, cache_stride
 #define KX_MFMA_BY_M(KS)                                                             \
     do {                                                                             \
         if (M <= 2) launch_awq_gemv_mfma<4, KS, 2, 1, PRO, EPI>(KX_MARGS);           \
@@ -762,7 +763,7 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
     if (act_ld < K) return KX_ERR_BAD_SHAPE;
     if (rows > 1) {
         // several rows: the matrix-core kernel, which produces activations 16 bytes at a time
-        if (d->in_kind == KX_IN_ATTN || d->out_kind == KX_OUT_QKV_ROPE) return KX_ERR_BAD_SHAPE;
+        if (d->in_kind == KX_IN_ATTN) return KX_ERR_BAD_SHAPE;
         if (!kx::mfma_shape_ok(N, group_size) || (act_ld % 8) != 0) return KX_ERR_BAD_SHAPE;
     }
 
@@ -860,6 +861,10 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
                 (d->rope_n_q_heads + 2 * d->rope_n_kv_heads) % (kx::kTileCols / kx::kHeadDim) != 0) {
                 return KX_ERR_BAD_SHAPE;
             }
+            // several rows are several sequences, each with a cache pair of its own
+            if (rows > 1 && d->cache_stride < static_cast<size_t>(d->cache_positions) * d->rope_n_kv_heads * kx::kHeadDim) {
+                return KX_ERR_BAD_SHAPE;
+            }
             rope = kx::RopeTarget{d->q_gain, d->k_gain, d->q_out, d->k_cache, d->v_cache, d->pos, d->cache_positions,
                                   d->rope_n_q_heads, d->rope_n_kv_heads, log2f(d->rope_theta), d->qk_eps};
             out_probe = d->q_out;
@@ -878,11 +883,12 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
         rc = kx::resolve_workspace(mp, rows, N, workspace, workspace_bytes, &partials, &counters);
         if (rc != KX_OK) return rc;
         hipStream_t s = kx::as_stream(stream);
-#define KX_MCHAIN(PRO, EPI) kx::launch_mfma_fused<PRO, EPI>(mp, fi, res, x, qweight, scales, qzeros, y, partials, counters, rows, K, N, group_size, s)
-#define KX_MBY_OUT(PRO)                                                       \
-    do {                                                                      \
-        if (d->out_kind == KX_OUT_ROW) KX_MCHAIN(PRO, kx::kEpiStore);         \
-        else KX_MCHAIN(PRO, kx::kEpiResidual);                                \
+#define KX_MCHAIN(PRO, EPI) kx::launch_mfma_fused<PRO, EPI>(mp, fi, res, x, qweight, scales, qzeros, y, partials, counters, rows, K, N, group_size, s, rope, d->cache_stride)
+#define KX_MBY_OUT(PRO)                                                               \
+    do {                                                                              \
+        if (d->out_kind == KX_OUT_ROW) KX_MCHAIN(PRO, kx::kEpiStore);                 \
+        else if (d->out_kind == KX_OUT_RESIDUAL) KX_MCHAIN(PRO, kx::kEpiResidual);    \
+        else KX_MCHAIN(PRO, kx::kEpiQkRope);                                          \
     } while (0)
         switch (d->in_kind) {
             case KX_IN_ROW: KX_MBY_OUT(kx::kProNone); break;

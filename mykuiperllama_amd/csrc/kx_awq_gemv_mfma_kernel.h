@@ -32,6 +32,7 @@
 
 #include "kx_common.h"
 #include "kx_gemv_fused.h"
+#include "kx_rope.h"
 #include "kx_splitk_exchange.h"
 
 namespace kx {
@@ -80,14 +81,15 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group_shift, int ktiles, FusedInput fi, ResidualTarget res) {
+    int M, int K, int N, int group_shift, int ktiles, FusedInput fi, ResidualTarget res, RopeTarget rope,
+    size_t cache_stride) {
     constexpr int WROWS = KS * kStepRows;  // rows of K per wave
     constexpr int KB = WAVES * WROWS;      // rows of K per workgroup
     constexpr int ROWS = MC * ROUNDS;      // activation rows this kernel carries (>= M)
     constexpr int THREADS = WAVES * kWave;
     static_assert(THREADS >= kTileCols, "one thread per tile column");
     static_assert(PRO == kProNone || PRO == kProSwiGLU || PRO == kProPreNorm, "prologues of the matrix-core kernel");
-    static_assert(EPI == kEpiStore || EPI == kEpiResidual, "epilogues of the matrix-core kernel");
+    static_assert(EPI == kEpiStore || EPI == kEpiResidual || EPI == kEpiQkRope, "epilogues of the matrix-core kernel");
     constexpr bool STAGED = PRO != kProNone;
     // A staged row is the workgroup's K range plus 16 bytes, so that the rows a wave reads together
     // start in different banks.
@@ -112,6 +114,29 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
     const int nw = N >> 3;
 
     const int kwave = kt * KB + wave * WROWS;  // first row of this wave
+
+    // The rotary epilogue (row m of the result belongs to sequence m): the workgroup that finishes a column
+    // tile holds two heads of every row; wave w will take the (row, head) items w, w + WAVES, ...  Its
+    // positions and the heads' gains are requested now, long before the epilogue needs them.
+    constexpr int ROPE_ITEMS = (2 * ROWS + WAVES - 1) / WAVES;  // items per wave
+    int rope_pos[EPI == kEpiQkRope ? ROPE_ITEMS : 1];
+    uint16_t rope_ga[2], rope_gb[2];
+    if constexpr (EPI == kEpiQkRope) {
+#pragma unroll
+        for (int i = 0; i < ROPE_ITEMS; i++) {
+            const int r = (wave + i * WAVES) / 2;
+            rope_pos[i] = rope.pos[r < M ? r : M - 1];
+        }
+        // both gains, then a select of values (a select between pointers ends up as a table in private memory)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const bool q_head = ct * (kTileCols / kHeadDim) + h < rope.n_q;
+            const uint16_t qa = rope.q_gain[lane], qb = rope.q_gain[lane + 64];
+            const uint16_t ka = rope.k_gain[lane], kb = rope.k_gain[lane + 64];
+            rope_ga[h] = q_head ? qa : ka;
+            rope_gb[h] = q_head ? qb : kb;
+        }
+    }
 
     // ---- operands of the activation prologue go out first: they are small, mostly cached, and the prologue
     // should run while the weights are still on their way ----
@@ -352,15 +377,17 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         return;
     }
 #endif
-    if constexpr (EPI == kEpiResidual) {
-        static_assert(THREADS == kTileCols, "the residual epilogue is laid out for 256 threads");
+    if constexpr (EPI == kEpiResidual || EPI == kEpiQkRope) {
+        static_assert(THREADS == kTileCols, "these epilogues are laid out for 256 threads");
         // Thread t ends up with the finished sums of tile column t, every row; the residual rows are
         // requested as soon as the workgroup knows that it is the one to finish.
         float sum[ROWS];
-        uint16_t rin[ROWS];
+        uint16_t rin[EPI == kEpiResidual ? ROWS : 1];
         auto load_residual = [&] {
+            if constexpr (EPI == kEpiResidual) {
 #pragma unroll
-            for (int r = 0; r < ROWS; r++) rin[r] = res.in[static_cast<size_t>(r < M ? r : M - 1) * N + own_ld];
+                for (int r = 0; r < ROWS; r++) rin[r] = res.in[static_cast<size_t>(r < M ? r : M - 1) * N + own_ld];
+            }
         };
         if constexpr (ROWS >= 4) {
             // the wide read-back hands out two columns and half of the rows per thread: through LDS (the
@@ -391,24 +418,47 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
             if (!splitk_exchange_sum<ROWS>(psum, sum, 0, M, N, ct, kt, ktiles, ct, partials, counters, &s_prev)) return;
             load_residual();
         }
-        __shared__ float s_quarter[ROWS][kTileCols / kWave];
-        const bool col_ok = own_col < N;
+        if constexpr (EPI == kEpiQkRope) {
+            // The finished rows, rounded to bf16 as a separate GEMV would store them, go through LDS so that a
+            // wave holds elements i and i + 64 of a head in lane i, the layout of the per-head routine.
+            __shared__ uint16_t s_rows[ROWS][kTileCols];
 #pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            float rv = 0.0f;
-            if (col_ok && r < M) {
-                const float o = bf16_to_f32(f32_to_bf16(sum[r]));  // the projection's output is a bf16 tensor
-                const uint16_t rbits = f32_to_bf16(bf16_to_f32(rin[r]) + o);
-                res.out[static_cast<size_t>(r) * N + own_col] = rbits;
-                rv = bf16_to_f32(rbits);
+            for (int r = 0; r < ROWS; r++) s_rows[r][tid] = f32_to_bf16(sum[r]);
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < ROPE_ITEMS; i++) {
+                const int item = wave + i * WAVES;
+                const int r = item / 2;
+                const int h = item % 2;
+                if (r < M) {  // the same in every lane of the wave
+                    RopeTarget t = rope;
+                    t.q_out += static_cast<size_t>(r) * rope.n_q * kHeadDim;
+                    t.k_cache += static_cast<size_t>(r) * cache_stride;
+                    t.v_cache += static_cast<size_t>(r) * cache_stride;
+                    qk_norm_rope_head_with(s_rows[r][h * kHeadDim + lane], s_rows[r][h * kHeadDim + lane + 64],
+                                           ct * (kTileCols / kHeadDim) + h, lane, t, rope_pos[i], rope_ga[h], rope_gb[h]);
+                }
             }
-            const float q = wave_sum(rv * rv);
-            if (lane == 0) s_quarter[r][wave] = q;
-        }
-        __syncthreads();
-        if (tid < M) {
-            res.sumsq[static_cast<size_t>(tid) * gridDim.x + ct] =
-                ((s_quarter[tid][0] + s_quarter[tid][1]) + s_quarter[tid][2]) + s_quarter[tid][3];
+        } else {
+            __shared__ float s_quarter[ROWS][kTileCols / kWave];
+            const bool col_ok = own_col < N;
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                float rv = 0.0f;
+                if (col_ok && r < M) {
+                    const float o = bf16_to_f32(f32_to_bf16(sum[r]));  // the projection's output is a bf16 tensor
+                    const uint16_t rbits = f32_to_bf16(bf16_to_f32(rin[r]) + o);
+                    res.out[static_cast<size_t>(r) * N + own_col] = rbits;
+                    rv = bf16_to_f32(rbits);
+                }
+                const float q = wave_sum(rv * rv);
+                if (lane == 0) s_quarter[r][wave] = q;
+            }
+            __syncthreads();
+            if (tid < M) {
+                res.sumsq[static_cast<size_t>(tid) * gridDim.x + ct] =
+                    ((s_quarter[tid][0] + s_quarter[tid][1]) + s_quarter[tid][2]) + s_quarter[tid][3];
+            }
         }
     } else if constexpr (ROWS >= 4) {
         static_assert(THREADS == kTileCols, "the wide exchange is laid out for 256 threads");
@@ -423,13 +473,14 @@ inline void launch_awq_gemv_mfma(const uint16_t* x, const int32_t* qweight, cons
                                  const int32_t* qzeros, uint16_t* y, float* partials, uint32_t* counters,
                                  int M, int K, int N, int group_shift, int coltiles, int ktiles,
                                  hipStream_t stream, const FusedInput& fi = FusedInput{},
-                                 const ResidualTarget& res = ResidualTarget{}) {
+                                 const ResidualTarget& res = ResidualTarget{}, const RopeTarget& rope = RopeTarget{},
+                                 size_t cache_stride = 0) {
     dim3 grid(coltiles, ktiles, 1);
     dim3 block(WAVES * kWave, 1, 1);
     hipLaunchKernelGGL((awq_gemv_mfma_kernel<WAVES, KS, MC, ROUNDS, PRO, EPI>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group_shift, ktiles, fi, res);
+                       group_shift, ktiles, fi, res, rope, cache_stride);
 }
 
 }  // namespace kx

@@ -270,17 +270,23 @@ class BatchDecodeModel:
     sequence ([B, positions, n_kv, 128] per layer) and activations of B rows.  The GEMVs run on the matrix-core
     kernel (2 <= B <= 16 rows), rotation and attention take the sequence as a grid dimension.
 
-    fused=True   seven launches per layer: q|k|v with the RMSNorm on the way in, rotation + cache append,
-                 attention (two stages), o with the residual add on the way out, gate|up with the RMSNorm on
-                 the way in, down with SwiGLU on the way in and the residual add on the way out
+    fused=True   six or seven launches per layer: q|k|v with the RMSNorm on the way in (and, for up to four
+                 sequences, rotation + cache append on the way out; a launch of its own otherwise), attention
+                 (two stages), o with the residual add on the way out, gate|up with the RMSNorm on the way in,
+                 down with SwiGLU on the way in and the residual add on the way out
     fused=False  every operator a launch of its own (SwiGLU one per sequence)
     The two agree to the rounding of the RMSNorm's sum of squares (added per 256 columns when fused).
     """
 
-    def __init__(self, single, batch):
+    def __init__(self, single, batch, rope_in_qkv=None):
         torch = single.torch
         if not 2 <= batch <= 16:
             raise ValueError("2 <= batch <= 16")
+        # Rotation and cache append ride in the epilogue of the q|k|v GEMV for up to four sequences: the
+        # workgroup that finishes a column tile runs the per-head routine for two heads of every row, which
+        # takes longer than the launch it saves from eight rows on (measured, tokens/s at 2 / 8 / 16 sequences:
+        # 909 / 2243 / 3051 with the epilogue, 886 / 2254 / 3111 with the separate launch).
+        self.rope_in_qkv = batch <= 4 if rope_in_qkv is None else bool(rope_in_qkv)
         self.torch = torch
         self.cfg = c = single.cfg
         self.batch = B = batch
@@ -372,14 +378,24 @@ class BatchDecodeModel:
         into_residual = {"out_kind": capi.OUT_RESIDUAL, "residual_in": x, "residual_out": x, "sumsq_out": ssq, "rows": B}
         for li, L in enumerate(self.layers):
             qw, sc, qz = L["qkv"]
+            if self.rope_in_qkv:
+                out = {"out_kind": capi.OUT_QKV_ROPE, "q_out": self.q, "pos": self.pos, "rope_n_q_heads": c.n_q,
+                       "rope_n_kv_heads": c.n_kv, "rope_theta": c.rope_theta, "qk_eps": c.eps, "q_gain": L["q_norm"],
+                       "k_gain": L["k_norm"], "k_cache": self.k_cache[li], "v_cache": self.v_cache[li],
+                       "cache_positions": self.max_positions, "cache_stride": self.k_cache[li].stride(0), "rows": B}
+            else:
+                out = {"out_kind": capi.OUT_ROW, "y": self.qkv, "rows": B}
             if li == 0:  # the embedding rows come without their sums of squares
                 capi.rmsnorm_bf16(x, L["in_norm"], self.h, c.eps)
-                self._awq(self.h, L["qkv"], self.qkv)
+                capi.gemv_awq_chain_bf16(dict(out, in_kind=capi.IN_ROW, x=self.h), qw, sc, qz, H, c.qkv_out, g, ws)
             else:
-                capi.gemv_awq_chain_bf16({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": ssq, "norm_parts": parts,
-                                          "norm_gain": L["in_norm"], "norm_eps": c.eps, "out_kind": capi.OUT_ROW,
-                                          "y": self.qkv, "rows": B}, qw, sc, qz, H, c.qkv_out, g, ws)
-            self._attention(li, L)
+                capi.gemv_awq_chain_bf16(dict(out, in_kind=capi.IN_NORM, norm_row=x, norm_sumsq=ssq, norm_parts=parts,
+                                              norm_gain=L["in_norm"], norm_eps=c.eps), qw, sc, qz, H, c.qkv_out, g, ws)
+            if not self.rope_in_qkv:
+                capi.qk_norm_rope_batch_bf16(self.qkv, L["q_norm"], L["k_norm"], self.q, self.k_cache[li],
+                                             self.v_cache[li], c.n_q, c.n_kv, self.pos, c.rope_theta, c.eps)
+            capi.attn_decode_batch_bf16(self.q, self.k_cache[li], self.v_cache[li], self.attn, c.n_q, c.n_kv, self.pos,
+                                        self.max_positions, self.attn_ws)
             qw, sc, qz = L["o"]
             capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_ROW, x=self.attn),
                                      qw, sc, qz, c.n_q * c.head_dim, H, g, ws)
@@ -394,7 +410,7 @@ class BatchDecodeModel:
         return self._head(with_lm_head)
 
     def launches_per_step(self, with_lm_head=True, fused=True):
-        per_layer = 7 if fused else 10 + self.batch
+        per_layer = (6 if self.rope_in_qkv else 7) if fused else 10 + self.batch
         return 1 + self.cfg.layers * per_layer + (1 if fused else 0) + 1 + (2 if with_lm_head else 0)
 
 

@@ -120,7 +120,7 @@ def test_batched_step_matches_one_sequence_models(capi, torch, B):
     cfg = decode.ModelConfig(layers=2, hidden=1024, intermediate=3072, n_q=8, n_kv=2, vocab=2048)
     max_pos = 320
     single = decode.DecodeModel(cfg, max_pos)
-    batch = decode.BatchDecodeModel(single, B)
+    batch = decode.BatchDecodeModel(single, B, rope_in_qkv=(B != 16))  # both forms of the q|k|v launch
     lengths = [17 + 13 * b for b in range(B)]
     batch.prefill_cache_random(lengths)
     tokens = [(101 * b + 7) % cfg.vocab for b in range(B)]

@@ -196,6 +196,51 @@ def test_mlp_block_in_two_launches_matches_five(capi, torch, M):
     assert torch.allclose(sumsq_out.double(), tile_sums(torch, out), rtol=1e-5, atol=0)
 
 
+@pytest.mark.parametrize("K,n_q,n_kv,group", [(4096, 32, 8, 128), (5120, 64, 8, 128), (512, 4, 2, 32)])
+@pytest.mark.parametrize("M", ROWS)
+def test_rotary_output_equals_gemv_then_batched_rotation(capi, torch, K, n_q, n_kv, group, M):
+    """q|k|v projection of M sequences with per-head norm, rotation and cache append on the way out: bit for
+    bit the plain GEMV followed by kx_qk_norm_rope_batch_bf16 (row input), every sequence at its own position."""
+    heads = n_q + 2 * n_kv
+    N = heads * 128
+    max_pos = 96
+    qw, sc, qz = weights(torch, f"sb_rope_{K}_{N}", K, N, group)
+    ws = capi.make_workspace(M, K, N)
+    x = bf16_rand(torch, (M, K), 7 * M + K)
+    q_gain = bf16_rand(torch, (128,), 2, 0.1) + 1.0
+    k_gain = bf16_rand(torch, (128,), 3, 0.1) + 1.0
+    positions = [(29 * m + 5) % max_pos for m in range(M)]
+    positions[0], positions[-1] = 0, max_pos - 1
+    pos = torch.tensor(positions, dtype=torch.int32, device="cuda")
+    kc = bf16_rand(torch, (M, max_pos, n_kv, 128), 4)
+    vc = bf16_rand(torch, (M, max_pos, n_kv, 128), 5)
+    kc1, vc1 = kc.clone(), vc.clone()
+
+    qkv = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_bf16(x, qw, sc, qz, qkv, group, ws)
+    q_sep = torch.empty((M, n_q * 128), dtype=torch.bfloat16, device="cuda")
+    capi.qk_norm_rope_batch_bf16(qkv, q_gain, k_gain, q_sep, kc1, vc1, n_q, n_kv, pos, 1e6, 1e-6)
+
+    q = torch.full((M, n_q * 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_chain_bf16({"in_kind": capi.IN_ROW, "x": x, "out_kind": capi.OUT_QKV_ROPE, "q_gain": q_gain,
+                              "k_gain": k_gain, "q_out": q, "k_cache": kc, "v_cache": vc, "pos": pos,
+                              "rope_n_q_heads": n_q, "rope_n_kv_heads": n_kv, "rope_theta": 1e6, "qk_eps": 1e-6,
+                              "cache_positions": max_pos, "cache_stride": kc.stride(0), "rows": M},
+                             qw, sc, qz, K, N, group, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(bits(q, torch), bits(q_sep, torch))
+    assert torch.equal(bits(kc, torch), bits(kc1, torch))
+    assert torch.equal(bits(vc, torch), bits(vc1, torch))
+    # caches closer together than they are long are refused
+    with pytest.raises(capi.KxError) as e:
+        capi.gemv_awq_chain_bf16({"in_kind": capi.IN_ROW, "x": x, "out_kind": capi.OUT_QKV_ROPE, "q_gain": q_gain,
+                                  "k_gain": k_gain, "q_out": q, "k_cache": kc, "v_cache": vc, "pos": pos,
+                                  "rope_n_q_heads": n_q, "rope_n_kv_heads": n_kv, "rope_theta": 1e6, "qk_eps": 1e-6,
+                                  "cache_positions": max_pos, "cache_stride": kc.stride(0) - 128, "rows": M},
+                                 qw, sc, qz, K, N, group, ws)
+    assert e.value.code == -2
+
+
 def test_what_several_rows_refuse(capi, torch):
     K, N, group, M = 512, 256, 128, 4
     qw, sc, qz = weights(torch, "sb_refuse", K, N, group)
