@@ -117,6 +117,8 @@ int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight, const uin
  *       residual, delta bf16 [M,K] (16-byte aligned), gain bf16 [K]; r is written to residual_out
  *       [M,K] when that is not null.  residual_out must differ from residual and delta
  *       (KX_ERR_ALIAS): every workgroup reads the whole incoming row.  K <= 8192.
+ * These launches (and kx_gemv_awq_qkv_rope_bf16, kx_gemv_awq_attn_merge_bf16 and the chained launch with any
+ * input but KX_IN_ROW) address the packed weights with 32-bit offsets: K * N / 2 < 2^31, else KX_ERR_BAD_SHAPE.
  * Replaces: LayerSwiGLU + LayerMatmul, resp. LayerAdd + LayerRMSNorm + LayerMatmul, executed back
  * to back (slots kuiper/include/op/layer.h:8-20; none of the three is implemented in the reference).
  * ------------------------------------------------------------------------------------------ */

@@ -298,6 +298,11 @@ inline int check_awq_weights(const int32_t* qweight, const uint16_t* scales, con
     return KX_OK;
 }
 
+// The launches with an activation prologue address the packed weights with 32-bit offsets.
+inline bool weights_fit_buffer_loads(int K, int N) {
+    return static_cast<size_t>(K) * N / 2 < (static_cast<size_t>(1) << 31);
+}
+
 // Do the byte ranges [a, a + abytes) and [b, b + bbytes) share a byte?  Null pointers overlap nothing.
 inline bool ranges_overlap(const void* a, size_t abytes, const void* b, size_t bbytes) {
     if (!a || !b || abytes == 0 || bbytes == 0) return false;
@@ -548,6 +553,7 @@ extern "C" int kx_gemv_awq_swiglu_bf16(const uint16_t* gate, const uint16_t* up,
     if (!gate || !up) return KX_ERR_NULL_POINTER;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
     if (rc != KX_OK) return rc;
+    if (!kx::weights_fit_buffer_loads(K, N)) return KX_ERR_BAD_SHAPE;
     if (act_ld < K) return KX_ERR_BAD_SHAPE;
     if (reinterpret_cast<uintptr_t>(gate) % 2 || reinterpret_cast<uintptr_t>(up) % 2) return KX_ERR_ALIGNMENT;
     kx::FusedInput fi{};
@@ -585,6 +591,7 @@ extern "C" int kx_gemv_awq_addnorm_bf16(const uint16_t* residual, const uint16_t
     if (!residual || !gain) return KX_ERR_NULL_POINTER;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
     if (rc != KX_OK) return rc;
+    if (!kx::weights_fit_buffer_loads(K, N)) return KX_ERR_BAD_SHAPE;
     if (reinterpret_cast<uintptr_t>(residual) % 16 || reinterpret_cast<uintptr_t>(delta) % 16 ||
         reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
         return KX_ERR_ALIGNMENT;
@@ -642,6 +649,7 @@ extern "C" int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_
     const int N = (n_q_heads + 2 * n_kv_heads) * kx::kHeadDim;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, q_out, 1, K, N, group_size);
     if (rc != KX_OK) return rc;
+    if (!kx::weights_fit_buffer_loads(K, N)) return KX_ERR_BAD_SHAPE;
     if (reinterpret_cast<uintptr_t>(residual) % 16 || reinterpret_cast<uintptr_t>(delta) % 16 ||
         reinterpret_cast<uintptr_t>(gain) % 2 || reinterpret_cast<uintptr_t>(residual_out) % 2) {
         return KX_ERR_ALIGNMENT;
@@ -692,6 +700,7 @@ extern "C" int kx_gemv_awq_attn_merge_bf16(const void* attn_workspace, size_t at
     const int K = n_q_heads * kx::kHeadDim;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, 1, K, N, group_size);
     if (rc != KX_OK) return rc;
+    if (!kx::weights_fit_buffer_loads(K, N)) return KX_ERR_BAD_SHAPE;
     const int nchunks = kx::attn_chunks_of(max_positions);
     // a thread holds kMergeHold values of each of its elements: longer contexts take the separate merge
     if (nchunks > kx::kMergeParts * kx::kMergeHold) return KX_ERR_BAD_SHAPE;
@@ -874,6 +883,7 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
     // 8-byte alignment is what the plain store asks of y; the other outputs are written per element
     int rc = kx::check_awq_weights(qweight, scales, qzeros, out_probe, rows, K, N, group_size, d->out_kind == KX_OUT_ROW);
     if (rc != KX_OK) return rc;
+    if (d->in_kind != KX_IN_ROW && !kx::weights_fit_buffer_loads(K, N)) return KX_ERR_BAD_SHAPE;
     if (d->in_kind == KX_IN_ATTN && (K % kx::kHeadDim) != 0) return KX_ERR_BAD_SHAPE;
 
     if (rows > 1) {
