@@ -85,7 +85,7 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
 
 /* kx_gemv_awq_bf16 for callers that cannot allocate or hand over a workspace (code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc): the split-K workspace is a static device array inside
- * the library, kx_gemv_awq_static_scratch_bytes() bytes (64 KiB of counters + 8 MiB of partial sums) per GPU
+ * the library, kx_gemv_awq_static_scratch_bytes() bytes (256 KiB of counters + 8 MiB of partial sums) per GPU
  * the library runs on, held until the process ends.  Same arguments, kernels and bits as kx_gemv_awq_bf16.
  * A shape whose kx_gemv_workspace_bytes(M, K, N) exceeds the array is rejected with KX_ERR_WORKSPACE and
  * nothing is launched (every Qwen3-8B and -32B projection fits at M = 1, the 8B ones up to M = 4).

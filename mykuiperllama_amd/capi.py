@@ -158,7 +158,7 @@ def workspace_bytes(M, K, N):
 def make_workspace(M, K, N, device="cuda"):
     """Allocate and initialise a workspace large enough for a GEMV of this shape."""
     import torch
-    nbytes = max(workspace_bytes(M, K, N), 65536)
+    nbytes = max(workspace_bytes(M, K, N), 262144)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
     _check(load().kx_workspace_init(ws.data_ptr(), nbytes, _stream()))
     return ws

@@ -16,9 +16,11 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // Workspace layout: [kCounterBytes of arrival counters, one per 64-byte line][fp32 partial sums].
 // Counters that share a line serialise at the memory side (~10 ns per atomic, measured), so
-// every (column tile, activation tile) pair gets a line of its own.
-constexpr size_t kCounterBytes = 65536;
-constexpr int kMaxTiles = kCounterBytes / 64;
+// every (column tile, activation tile) pair gets lines of its own: four of them, one per quarter of
+// the tile, for the exchange in which every wave of 64 columns reports for itself.
+constexpr int kCountersPerTile = 4;
+constexpr size_t kCounterBytes = 262144;
+constexpr int kMaxTiles = kCounterBytes / 64 / kCountersPerTile;
 
 // nibble i of a packed word holds column 8j + kOrder[i]
 __host__ __device__ constexpr int order_of(int i) {

@@ -179,7 +179,7 @@ def test_bad_arguments_are_rejected_before_launch(capi, torch):
     L = capi.load()
     s = torch.cuda.current_stream().cuda_stream
     args = (x.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), y.data_ptr())
-    small = torch.empty(65536 + 64, dtype=torch.uint8, device="cuda")
+    small = torch.empty(262144 + 64, dtype=torch.uint8, device="cuda")
     assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 128, None, 0, s) == -3     # K is split: needs a workspace
     assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 128, small.data_ptr(), small.numel(), s) == -3  # too small
     assert L.kx_gemv_awq_bf16(*args, 0, 1024, 64, 128, None, 0, s) == -2     # M = 0
@@ -189,7 +189,7 @@ def test_bad_arguments_are_rejected_before_launch(capi, torch):
     assert L.kx_gemv_awq_bf16(*args, 1, 1024, 64, 48, None, 0, s) == -2      # group not a multiple of 32
     assert L.kx_gemv_awq_bf16(None, *args[1:], 1, 1024, 64, 128, None, 0, s) == -1
     assert L.kx_gemv_awq_bf16(args[0] + 2, *args[1:], 1, 1024, 64, 128, None, 0, s) == -4  # x misaligned
-    assert capi.workspace_bytes(1, 1024, 64) > 65536
+    assert capi.workspace_bytes(1, 1024, 64) > 262144
     assert capi.workspace_bytes(0, 1024, 64) == 0
     torch.cuda.synchronize()
 

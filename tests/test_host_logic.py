@@ -75,8 +75,8 @@ def test_abi_version_and_error_strings(lib):
 
 
 def test_workspace_size_query(lib):
-    assert lib.kx_gemv_workspace_bytes(1, 4096, 4096) >= 65536 + (4096 // 256) * 4096 * 4
-    assert lib.kx_gemv_workspace_bytes(16, 12288, 4096) >= 65536 + 16 * (12288 // 256) * 4096 * 4
+    assert lib.kx_gemv_workspace_bytes(1, 4096, 4096) >= 262144 + (4096 // 256) * 4096 * 4
+    assert lib.kx_gemv_workspace_bytes(16, 12288, 4096) >= 262144 + 16 * (12288 // 256) * 4096 * 4
     assert lib.kx_gemv_workspace_bytes(0, 4096, 4096) == 0
     assert lib.kx_gemv_workspace_bytes(17, 4096, 4096) == 0
 

@@ -40,7 +40,7 @@ def _both(capi, torch, name, M, K, N):
 
 def test_static_scratch_entry_point_matches_the_workspace_entry_point(capi, torch, oracle):
     print("no-alloc entry point: 12288x4096 M=1, then 1024x512 M=2, then 4096x12288 M=3", flush=True)
-    assert capi.load().kx_gemv_awq_static_scratch_bytes() == 65536 + (8 << 20)
+    assert capi.load().kx_gemv_awq_static_scratch_bytes() == 262144 + (8 << 20)
     # two calls in a row on the shared array, the second one smaller, a third one on the MFMA kernel
     for name, M, K, N in (("static_a", 1, 12288, 4096), ("static_b", 2, 1024, 512), ("static_c", 3, 4096, 12288)):
         p, want, got = _both(capi, torch, name, M, K, N)
