@@ -510,10 +510,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     }
 #endif
     if constexpr (EPI == kEpiStore && MB == 1) {
-        // one activation row (m0 = blockIdx.y, M rows of N apart): every wave reports for itself
-        splitk_exchange_store_per_wave(psum[0], N, ct, kt, ktiles, blockIdx.y * coltiles + ct,
-                                       static_cast<size_t>(M) * N, partials + static_cast<size_t>(m0) * N, counters,
-                                       y + static_cast<size_t>(m0) * N);
+        // one activation row (MB == 1 is M == 1 in every plan): every wave reports for itself
+        splitk_exchange_store_per_wave(psum[0], N, ct, kt, ktiles, ct, partials, counters, y);
     } else if constexpr (EPI == kEpiStore) {
         splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
                                   &s_prev);

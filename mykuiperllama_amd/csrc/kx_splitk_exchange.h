@@ -172,8 +172,7 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
 // Qwen3-8B projections: 0.3-0.4 us per launch, 5.5 % on the step.
 // Called by every thread; `psum` as in splitk_exchange_sum (thread tid < 256 owns tile column tid).
 __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N, int ct, int kt, int ktiles,
-                                                               int counter_index, size_t tstride,
-                                                               float* __restrict__ partials,
+                                                               int counter_index, float* __restrict__ partials,
                                                                uint32_t* __restrict__ counters,
                                                                uint16_t* __restrict__ y) {
     const int tid = threadIdx.x;
@@ -184,7 +183,7 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
         if (col_ok) y[col] = f32_to_bf16(psum);
         return;
     }
-    // `partials` and `y` point at the activation row; tstride = floats between consecutive K tiles
+    const size_t tstride = static_cast<size_t>(N);  // floats between consecutive K tiles: one activation row
     if (col_ok) store_agent(partials + static_cast<size_t>(kt) * tstride + col, psum);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
@@ -196,28 +195,51 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
 
     // last of its quarter: every other wave's partial sums were acknowledged before its increment
     constexpr int TB = 16;
-    const bool two_runs = ktiles > TB && blockDim.x >= 2 * kTileCols;  // where splitk_exchange_sum has helpers
-    const int step = two_runs ? 2 : 1;
     const unsigned hcol = static_cast<unsigned>(col_ok ? col : N - 1);
-    float run[2] = {0.0f, 0.0f};
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        if (h == 1 && !two_runs) break;
-        for (int t0 = h; t0 < ktiles; t0 += TB * step) {
+    float sum = 0.0f;
+    if (!(ktiles > TB && blockDim.x >= 2 * kTileCols)) {
+        for (int t0 = 0; t0 < ktiles; t0 += TB) {
             float v[TB];
 #pragma unroll
             for (int u = 0; u < TB; u++) {
                 // clamped address, masked value: the loads of a batch are straight-line code
-                const int t = t0 + u * step;
+                const int t = t0 + u;
                 const int tc = t < ktiles ? t : ktiles - 1;
                 const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
                 v[u] = t < ktiles ? got : 0.0f;
             }
 #pragma unroll
-            for (int u = 0; u < TB; u++) run[h] += v[u];
+            for (int u = 0; u < TB; u++) sum += v[u];
         }
+    } else {
+        // where splitk_exchange_sum has helper threads: the even tiles in order, the odd ones likewise, even + odd
+        float odd = 0.0f;
+        for (int t0 = 0; t0 < ktiles; t0 += 2 * TB) {
+            float v[TB];
+#pragma unroll
+            for (int u = 0; u < TB; u++) {
+                const int t = t0 + 2 * u;
+                const int tc = t < ktiles ? t : ktiles - 1;
+                const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
+                v[u] = t < ktiles ? got : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < TB; u++) sum += v[u];
+        }
+        for (int t0 = 1; t0 < ktiles; t0 += 2 * TB) {
+            float v[TB];
+#pragma unroll
+            for (int u = 0; u < TB; u++) {
+                const int t = t0 + 2 * u;
+                const int tc = t < ktiles ? t : ktiles - 1;
+                const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
+                v[u] = t < ktiles ? got : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < TB; u++) odd += v[u];
+        }
+        sum += odd;
     }
-    const float sum = two_runs ? run[0] + run[1] : run[0];
     if (col_ok) y[col] = f32_to_bf16(sum);
     if (tid % kWave == 0) {
         // leave the workspace ready for the next launch
