@@ -162,19 +162,22 @@ int kx_gemv_awq_qkv_rope_bf16(const uint16_t* residual, const uint16_t* delta, c
  *                                                        of kx_attn_decode_partial_bf16 (K = n_q_heads * 128)
  *   KX_IN_NORM      norm_row, norm_sumsq, norm_parts, norm_gain, norm_eps
  *                                                        x = gain * bf16(row * rsqrt(sum(sumsq) / K + eps)),
- *                                                        sumsq = the per-tile sums KX_OUT_RESIDUAL left
+ *                                                        sumsq = what KX_OUT_RESIDUAL left: float [norm_parts, 4],
+ *                                                        norm_parts = ceil(K / 256), 16-byte aligned
  *   KX_OUT_ROW      y                                    y = bf16(o)
  *   KX_OUT_RESIDUAL residual_in, residual_out, sumsq_out residual_out = bf16(residual_in + bf16(o)) (may be
- *                                                        in place), sumsq_out[t] = sum of squares of columns
- *                                                        256 t .. 256 t + 255 of residual_out, t < ceil(N / 256)
+ *                                                        in place), sumsq_out[t, i] = sum of squares of columns
+ *                                                        256 t + 64 i .. + 63 of residual_out: float
+ *                                                        [ceil(N / 256), 4] (quarters past N: 0)
  *   KX_OUT_QKV_ROPE q_gain, k_gain, q_out, k_cache, v_cache, pos, rope_n_q_heads, rope_n_kv_heads,
  *                   cache_positions, rope_theta, qk_eps  as kx_gemv_awq_qkv_rope_bf16 (N = (n_q + 2 n_kv) * 128)
  *
- * The sum of squares of KX_OUT_RESIDUAL / KX_IN_NORM is added tile by tile, an order of its own:
+ * The sum of squares of KX_OUT_RESIDUAL / KX_IN_NORM is added quarter by quarter and tile by tile
+ * (((Q0 + Q1) + Q2) + Q3 per tile, then the tiles), an order of its own:
  * results agree with kx_add_rmsnorm_bf16 followed by the GEMV to within the rounding of that sum
  * (an occasional last-bit difference in the normalised row), not bit for bit.
  * With rows = 2 .. KX_MAX_BATCH every tensor gains a leading dimension (x [rows, K], y / residual_* [rows, N],
- * norm_sumsq [rows, norm_parts], sumsq_out [rows, ceil(N / 256)]); gate, up and norm_row may have their rows
+ * norm_sumsq [rows, norm_parts, 4], sumsq_out [rows, ceil(N / 256), 4]); gate, up and norm_row may have their rows
  * act_ld elements apart.  That form runs on the matrix-core kernel and takes KX_IN_ROW / KX_IN_SWIGLU /
  * KX_IN_NORM with any output kind (KX_OUT_QKV_ROPE: q_out [rows, n_q * 128], pos [rows], one cache pair per
  * row, see cache_stride), a power-of-two group size, N a multiple of 16, act_ld a

@@ -812,9 +812,9 @@ extern "C" int kx_gemv_awq_chain_bf16(const kx_chain_desc* d, const int32_t* qwe
         case KX_IN_NORM:
             if (!d->norm_row || !d->norm_sumsq || !d->norm_gain) return KX_ERR_NULL_POINTER;
             if (d->norm_parts != (K + kx::kTileCols - 1) / kx::kTileCols || d->norm_parts > kx::kWave) return KX_ERR_BAD_SHAPE;
-            if (reinterpret_cast<uintptr_t>(d->norm_row) % 2 || reinterpret_cast<uintptr_t>(d->norm_sumsq) % 4 ||
+            if (reinterpret_cast<uintptr_t>(d->norm_row) % 2 || reinterpret_cast<uintptr_t>(d->norm_sumsq) % 16 ||
                 reinterpret_cast<uintptr_t>(d->norm_gain) % 2) {
-                return KX_ERR_ALIGNMENT;
+                return KX_ERR_ALIGNMENT;  // the four quarter sums of a tile are read as one 16-byte piece
             }
             if (rows > 1 && (!kx::aligned_to(d->norm_row, 16) || !kx::aligned_to(d->norm_gain, 16))) return KX_ERR_ALIGNMENT;
             fi.a = d->norm_row;

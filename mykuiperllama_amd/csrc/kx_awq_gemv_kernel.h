@@ -150,7 +150,9 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     float tile_ss = 0.0f;
     if constexpr (PRO == kProPreNorm) {
         const int part = tid % kWave;
-        tile_ss = fi.sumsq[part < fi.sumsq_parts ? part : fi.sumsq_parts - 1];
+        // four quarter sums per tile, added in the order that defines the tile's sum
+        const f32x4 qs = reinterpret_cast<const f32x4*>(fi.sumsq)[part < fi.sumsq_parts ? part : fi.sumsq_parts - 1];
+        tile_ss = ((qs.x + qs.y) + qs.z) + qs.w;
     }
 
     float acc[MB][8];
@@ -517,26 +519,20 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
                                   &s_prev);
     } else if constexpr (EPI == kEpiResidual) {
         static_assert(MB == 1, "the residual epilogue serves one activation row");
-        float sum[MB];
-        if (!splitk_exchange_sum<MB>(psum, sum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials,
-                                     counters, &s_prev)) {
-            return;
-        }
-        __shared__ float s_quarter[kTileCols / kWave];
+        // every wave of 64 columns finishes for itself (splitk_exchange_sum_per_wave) and leaves the sum of
+        // squares of its quarter of the tile: no barrier, no wave waits for another
+        float sum;
+        if (!splitk_exchange_sum_per_wave(psum[0], &sum, N, ct, kt, ktiles, ct, partials, counters)) return;
         const int col = ct * kTileCols + tid;
         float r = 0.0f;
-        if (tid < kTileCols && col < N) {
-            const float o = bf16_to_f32(f32_to_bf16(sum[0]));  // the projection's output is a bf16 tensor
+        if (col < N) {
+            const float o = bf16_to_f32(f32_to_bf16(sum));  // the projection's output is a bf16 tensor
             const uint16_t rbits = f32_to_bf16(bf16_to_f32(resid_pre) + o);
             res.out[col] = rbits;
             r = bf16_to_f32(rbits);
         }
-        if (tid < kTileCols) {
-            const float q = wave_sum(r * r);
-            if (lane == 0) s_quarter[tid / kWave] = q;
-        }
-        __syncthreads();
-        if (tid == 0) res.sumsq[ct] = ((s_quarter[0] + s_quarter[1]) + s_quarter[2]) + s_quarter[3];
+        const float q = wave_sum(r * r);
+        if (lane == 0) res.sumsq[ct * (kTileCols / kWave) + tid / kWave] = q;
     } else {
         static_assert(MB == 1, "the rotary epilogue serves one activation row");
         float sum[MB];

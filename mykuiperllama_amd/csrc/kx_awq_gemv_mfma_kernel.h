@@ -163,8 +163,9 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
             for (int rr = 0; rr < (ROWS + WAVES - 1) / WAVES; rr++) {
                 const int m = wave + rr * WAVES;
                 const int mc = m < M ? m : M - 1;
-                tile_ss[rr] = fi.sumsq[static_cast<size_t>(mc) * fi.sumsq_parts +
-                                       (lane < fi.sumsq_parts ? lane : fi.sumsq_parts - 1)];
+                const f32x4 qs = reinterpret_cast<const f32x4*>(fi.sumsq)[static_cast<size_t>(mc) * fi.sumsq_parts +
+                                                                          (lane < fi.sumsq_parts ? lane : fi.sumsq_parts - 1)];
+                tile_ss[rr] = ((qs.x + qs.y) + qs.z) + qs.w;  // the order that defines a tile's sum
             }
         }
     }
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
                 }
             }
         } else {
-            __shared__ float s_quarter[ROWS][kTileCols / kWave];
+            // a wave is a quarter of the tile: its sum of squares of every row goes out as it is
             const bool col_ok = own_col < N;
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
@@ -452,12 +453,9 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
                     rv = bf16_to_f32(rbits);
                 }
                 const float q = wave_sum(rv * rv);
-                if (lane == 0) s_quarter[r][wave] = q;
-            }
-            __syncthreads();
-            if (tid < M) {
-                res.sumsq[static_cast<size_t>(tid) * gridDim.x + ct] =
-                    ((s_quarter[tid][0] + s_quarter[tid][1]) + s_quarter[tid][2]) + s_quarter[tid][3];
+                if (lane == 0 && r < M) {
+                    res.sumsq[(static_cast<size_t>(r) * gridDim.x + ct) * (kTileCols / kWave) + wave] = q;
+                }
             }
         }
     } else if constexpr (ROWS >= 4) {

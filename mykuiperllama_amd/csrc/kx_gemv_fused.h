@@ -34,20 +34,21 @@ struct FusedInput {
     const float* part_ml;
     int nchunks;
     int heads_per_kv;
-    // kProPreNorm: sums of squares of the rows of `a`, [M, sumsq_parts], one partial per tile of 256 columns
-    // (at most 64)
+    // kProPreNorm: sums of squares of the rows of `a`, [M, sumsq_parts, 4]: per tile of 256 columns (at most
+    // 64 tiles) the sums of its four quarters of 64 columns, 16-byte aligned
     const float* sumsq;
     int sumsq_parts;
 };
 
 // kEpiResidual: the finished rows o are added to the residual stream, out = bf16(in + bf16(o)), and the
-// sum of squares of each new row is left per column tile for the RMSNorm that follows:
-//   sumsq[m, t] = ((Q0 + Q1) + Q2) + Q3,  Q_i = wave_sum over the 64 columns of quarter i of tile t
-// (kProPreNorm adds the tiles of a row with one more wave_sum, lane = tile).
+// sums of squares of each new row are left per quarter of a column tile for the RMSNorm that follows:
+//   sumsq[m, t, i] = Q_i = wave_sum over the 64 columns of quarter i of tile t
+// (kProPreNorm forms ((Q0 + Q1) + Q2) + Q3 per tile and adds the tiles of a row with one more wave_sum,
+// lane = tile).  A quarter is what one wave finishes, so no wave has to wait for another.
 struct ResidualTarget {
     const uint16_t* in;   // bf16 [M, N]
     uint16_t* out;        // bf16 [M, N], may be `in`: an element is read and written by the same thread
-    float* sumsq;         // [M, ceil(N / 256)]
+    float* sumsq;         // [M, ceil(N / 256), 4]
 };
 
 // What happens to the finished sums (EPI below).

@@ -171,18 +171,22 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
 // whose epilogues go through splitk_exchange_sum.  Measured against the workgroup-wide exchange on the seven
 // Qwen3-8B projections: 0.3-0.4 us per launch, 5.5 % on the step.
 // Called by every thread; `psum` as in splitk_exchange_sum (thread tid < 256 owns tile column tid).
-__device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N, int ct, int kt, int ktiles,
-                                                               int counter_index, float* __restrict__ partials,
-                                                               uint32_t* __restrict__ counters,
-                                                               uint16_t* __restrict__ y) {
+//
+// Returns true, the same in every lane of the wave, in the wave that ends up with the finished sums of its
+// 64 columns (`sum`); the other waves return false and are done.  Waves past the tile's 256 columns return
+// false at once.
+__device__ __forceinline__ bool splitk_exchange_sum_per_wave(float psum, float* sum_out, int N, int ct, int kt,
+                                                             int ktiles, int counter_index,
+                                                             float* __restrict__ partials,
+                                                             uint32_t* __restrict__ counters) {
     const int tid = threadIdx.x;
-    if (tid >= kTileCols) return;  // whole waves: the others own no column
+    if (tid >= kTileCols) return false;  // whole waves: the others own no column
+    if (ktiles == 1) {
+        *sum_out = psum;
+        return true;
+    }
     const int col = ct * kTileCols + tid;
     const bool col_ok = col < N;
-    if (ktiles == 1) {
-        if (col_ok) y[col] = f32_to_bf16(psum);
-        return;
-    }
     const size_t tstride = static_cast<size_t>(N);  // floats between consecutive K tiles: one activation row
     if (col_ok) store_agent(partials + static_cast<size_t>(kt) * tstride + col, psum);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -191,7 +195,7 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
     uint32_t prev = 0;
     if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
-    if (prev != static_cast<uint32_t>(ktiles - 1)) return;
+    if (prev != static_cast<uint32_t>(ktiles - 1)) return false;
 
     // last of its quarter: every other wave's partial sums were acknowledged before its increment
     constexpr int TB = 16;
@@ -240,11 +244,23 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
         }
         sum += odd;
     }
-    if (col_ok) y[col] = f32_to_bf16(sum);
+    *sum_out = sum;
     if (tid % kWave == 0) {
         // leave the workspace ready for the next launch
         __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    return true;
+}
+
+// The per-wave exchange followed by the plain epilogue: y[col] = bf16(sum).
+__device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N, int ct, int kt, int ktiles,
+                                                               int counter_index, float* __restrict__ partials,
+                                                               uint32_t* __restrict__ counters,
+                                                               uint16_t* __restrict__ y) {
+    float sum;
+    if (!splitk_exchange_sum_per_wave(psum, &sum, N, ct, kt, ktiles, counter_index, partials, counters)) return;
+    const int col = ct * kTileCols + static_cast<int>(threadIdx.x);
+    if (col < N) y[col] = f32_to_bf16(sum);
 }
 
 // The exchange for several activation rows (ROWS = 4, 8 or 16) and a workgroup of exactly 256 threads, more

@@ -120,7 +120,7 @@ class DecodeModel:
         self.act = buf(c.intermediate)
         self.down = buf(c.hidden)
         self.logits = buf(c.vocab)
-        self.ssq = torch.zeros(((c.hidden + 255) // 256,), dtype=torch.float32, device="cuda")
+        self.ssq = torch.zeros(((c.hidden + 255) // 256, 4), dtype=torch.float32, device="cuda")  # quarter sums per tile
         self.token = torch.zeros(1, dtype=torch.int32, device="cuda")
         self.pos = torch.zeros(1, dtype=torch.int32, device="cuda")
         self.next_token = torch.zeros(1, dtype=torch.int32, device="cuda")
@@ -230,7 +230,7 @@ class DecodeModel:
                                             c.rope_theta, c.eps, g, ws)
             else:
                 capi.gemv_awq_chain_bf16(dict(rope, in_kind=capi.IN_NORM, norm_row=x, norm_sumsq=ssq,
-                                              norm_parts=ssq.numel(), norm_gain=L["in_norm"], norm_eps=c.eps,
+                                              norm_parts=ssq.shape[0], norm_gain=L["in_norm"], norm_eps=c.eps,
                                               q_gain=L["q_norm"], k_gain=L["k_norm"], k_cache=self.k_cache[li],
                                               v_cache=self.v_cache[li]), qw, sc, qz, H, c.qkv_out, g, ws)
             qw, sc, qz = L["o"]
@@ -248,7 +248,7 @@ class DecodeModel:
                                          qw, sc, qz, c.n_q * c.head_dim, H, g, ws)
             qw, sc, qz = L["gateup"]
             capi.gemv_awq_chain_bf16({"in_kind": capi.IN_NORM, "norm_row": x, "norm_sumsq": ssq,
-                                      "norm_parts": ssq.numel(), "norm_gain": L["post_norm"], "norm_eps": c.eps,
+                                      "norm_parts": ssq.shape[0], "norm_gain": L["post_norm"], "norm_eps": c.eps,
                                       "out_kind": capi.OUT_ROW, "y": self.gu}, qw, sc, qz, H, 2 * I, g, ws)
             qw, sc, qz = L["down"]
             capi.gemv_awq_chain_bf16(dict(into_residual, in_kind=capi.IN_SWIGLU, gate=self.gu[:, :I],
@@ -311,7 +311,7 @@ class BatchDecodeModel:
         self.act = buf(c.intermediate)
         self.down = buf(c.hidden)
         self.logits = buf(c.vocab)
-        self.ssq = torch.zeros((B, (c.hidden + 255) // 256), dtype=torch.float32, device="cuda")
+        self.ssq = torch.zeros((B, (c.hidden + 255) // 256, 4), dtype=torch.float32, device="cuda")  # quarter sums per tile
         self.token = torch.zeros(B, dtype=torch.int32, device="cuda")
         self.pos = torch.zeros(B, dtype=torch.int32, device="cuda")
         self.next_token = torch.zeros(B, dtype=torch.int32, device="cuda")

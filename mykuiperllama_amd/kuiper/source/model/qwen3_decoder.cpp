@@ -135,7 +135,8 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
     attn_ = device_tensor(bf16, {c.n_q_heads * c.head_dim});
     gate_up_ = device_tensor(bf16, {2 * c.intermediate});
     logits_ = device_tensor(bf16, {c.vocab});
-    sumsq_ = device_tensor(base::DataType::DataTypeFp32, {(c.hidden + kTileColumns - 1) / kTileColumns});
+    // per 256 columns of the residual stream the sums of squares of its four quarters
+    sumsq_ = device_tensor(base::DataType::DataTypeFp32, {(c.hidden + kTileColumns - 1) / kTileColumns, 4});
     io_ = device_tensor(base::DataType::DataTypeInt32, {3});
 
     const int32_t big_k = std::max(std::max(c.hidden, c.intermediate), c.n_q_heads * c.head_dim);
@@ -401,7 +402,7 @@ int Qwen3Decoder::enqueue_step_fused() {
     const int32_t* pos = token + 1;
     int32_t* next = io_.ptr<int32_t>() + 2;
     const int32_t H = c.hidden, I = c.intermediate, QD = c.n_q_heads * c.head_dim, G = c.group_size;
-    const int32_t parts = static_cast<int32_t>(sumsq_.size());
+    const int32_t parts = sumsq_.get_dim(0);
 
     int rc = kx_embedding_bf16(u16(embed_), token, u16(x_), c.vocab, H, s);
     if (rc != KX_OK) return rc;

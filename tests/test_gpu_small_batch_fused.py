@@ -51,11 +51,12 @@ def rel_l2(a, b):
 
 
 def tile_sums(torch, rows):
-    """fp64 sums of squares per 256 columns of every row of a bf16 [M, N] tensor -> [M, ceil(N / 256)]."""
+    """fp64 sums of squares of every row of a bf16 [M, N] tensor per quarter (64 columns) of every tile of 256
+    columns -> [M, ceil(N / 256), 4]."""
     v = rows.double()
     pad = (-v.shape[1]) % 256
     v = torch.cat([v, torch.zeros((v.shape[0], pad), dtype=torch.float64, device=v.device)], dim=1)
-    return (v * v).view(v.shape[0], -1, 256).sum(dim=2)
+    return (v * v).view(v.shape[0], -1, 4, 64).sum(dim=3)
 
 
 # K, N, group: the Qwen3-8B down projection, a 32B-shaped one, a narrow one with a ragged last tile, groups of
@@ -103,14 +104,16 @@ def test_residual_output_equals_gemv_then_add(capi, torch, K, N, group, M, in_ki
     capi.add_bf16(resid, y, expected)
 
     parts = (N + 255) // 256
-    sumsq = torch.full((M, parts), float("nan"), dtype=torch.float32, device="cuda")
+    sumsq = torch.full((M, parts, 4), float("nan"), dtype=torch.float32, device="cuda")
     for in_place in (False, True):
         out = resid.clone() if in_place else torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
         desc.update({"residual_in": out if in_place else resid, "residual_out": out, "sumsq_out": sumsq})
         capi.gemv_awq_chain_bf16(desc, qw, sc, qz, K, N, group, ws)
         torch.cuda.synchronize()
         assert torch.equal(bits(out, torch), bits(expected, torch)), f"in_place={in_place}"
-        assert torch.allclose(sumsq.double(), tile_sums(torch, expected), rtol=1e-5, atol=0)
+        ref = tile_sums(torch, expected)
+        live = torch.arange(parts * 4, device="cuda").view(1, parts, 4).expand_as(ref) * 64 < N  # quarters with columns
+        assert torch.allclose(sumsq.double()[live], ref[live], rtol=1e-5, atol=0)
 
 
 @pytest.mark.parametrize("K,N,group", [(4096, 24576, 128), (5120, 10240, 128), (512, 272, 32), (1024, 512, 64)])
@@ -124,7 +127,7 @@ def test_norm_input_matches_the_fp32_restatement_and_the_one_row_launch(capi, to
     gain = bf16_rand(torch, (K,), K + 1, 0.5) + 1.0
     parts = (K + 255) // 256
     sumsq = tile_sums(torch, row).float().contiguous()
-    assert sumsq.shape == (M, parts)
+    assert sumsq.shape == (M, parts, 4)
 
     y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     desc = {"in_kind": capi.IN_NORM, "norm_row": row, "norm_sumsq": sumsq, "norm_parts": parts, "norm_gain": gain,
@@ -137,7 +140,7 @@ def test_norm_input_matches_the_fp32_restatement_and_the_one_row_launch(capi, to
     assert torch.equal(bits(y, torch), bits(again, torch))
 
     # the restatement: normalised row (bf16 rounding points as in the kernels), then the CPU oracle's GEMV
-    inv = torch.rsqrt(sumsq.double().sum(dim=1, keepdim=True) / K + EPS).float()
+    inv = torch.rsqrt(sumsq.double().sum(dim=(1, 2)).view(-1, 1) / K + EPS).float()
     h = (gain.float() * (row.float() * inv).bfloat16().float()).bfloat16()
     ref = oracle.gemv_awq_f64(H.bf16_bits(h, torch), p["qweight"], p["scales"], p["qzeros"], group)
     assert rel_l2(y.float().cpu(), torch.from_numpy(ref)) <= 2e-3
@@ -184,7 +187,7 @@ def test_mlp_block_in_two_launches_matches_five(capi, torch, M):
                               "norm_gain": gain, "norm_eps": EPS, "out_kind": capi.OUT_ROW, "y": gu2, "rows": M},
                              *gu_w, hidden, 2 * inter, group, ws)
     out = torch.empty_like(resid)
-    sumsq_out = torch.empty((M, parts), dtype=torch.float32, device="cuda")
+    sumsq_out = torch.empty((M, parts, 4), dtype=torch.float32, device="cuda")
     capi.gemv_awq_chain_bf16({"in_kind": capi.IN_SWIGLU, "gate": gu2[:, :inter], "up": gu2[:, inter:],
                               "act_ld": 2 * inter, "out_kind": capi.OUT_RESIDUAL, "residual_in": resid,
                               "residual_out": out, "sumsq_out": sumsq_out, "rows": M},
