@@ -535,22 +535,27 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         if (lane == 0) res.sumsq[ct * (kTileCols / kWave) + tid / kWave] = q;
     } else {
         static_assert(MB == 1, "the rotary epilogue serves one activation row");
-        float sum[MB];
-        if (!splitk_exchange_sum<MB>(psum, sum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials,
-                                     counters, &s_prev)) {
-            return;
-        }
-        // A column tile is two heads of 128.  The finished row, rounded to bf16 as a separate GEMV
-        // would store it, goes through LDS so that the first wave of each head holds elements i and
-        // i + 64 in lane i, the layout of the per-head routine.
-        __shared__ uint16_t s_row[kTileCols];
-        if (tid < kTileCols) s_row[tid] = f32_to_bf16(sum[0]);
-        __syncthreads();
-        if (tid < kTileCols && (tid & 64) == 0) {
-            const int local = tid >> 7;
-            const int head = ct * (kTileCols / kHeadDim) + local;
-            qk_norm_rope_head_with(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane, rope,
-                                   rope_pos, rope_gain_a, rope_gain_b);
+        // A column tile is two heads of 128 (the host admits whole tiles only).  The finished row is rounded
+        // to bf16 as a separate GEMV would store it; lane i of the finishing wave holds elements i and i + 64
+        // of its head, the layout of the per-head routine.
+        if (ktiles == 1) {
+            // no exchange: the two waves of a head meet in LDS
+            __shared__ uint16_t s_row[kTileCols];
+            if (tid < kTileCols) s_row[tid] = f32_to_bf16(psum[0]);
+            __syncthreads();
+            if (tid < kTileCols && (tid & 64) == 0) {
+                const int local = tid >> 7;
+                const int head = ct * (kTileCols / kHeadDim) + local;
+                qk_norm_rope_head_with(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane,
+                                       rope, rope_pos, rope_gain_a, rope_gain_b);
+            }
+        } else {
+            // the last of the head's waves over all K tiles finishes the head: no barrier, no LDS
+            float lo, hi;
+            if (!splitk_exchange_sum_per_head(psum[0], &lo, &hi, N, ct, kt, ktiles, partials, counters)) return;
+            const int head = ct * (kTileCols / kHeadDim) + (tid >> 7);
+            qk_norm_rope_head_with(f32_to_bf16(lo), f32_to_bf16(hi), head, lane, rope, rope_pos, rope_gain_a,
+                                   rope_gain_b);
         }
     }
 }

@@ -263,6 +263,82 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
     if (col < N) y[col] = f32_to_bf16(sum);
 }
 
+// Sums of the partial sums of columns `col` and `col + 64` over K tiles t_begin, t_begin + STEP, ... below
+// `ktiles`, added to `a` and `b` in that order; batches of sixteen K tiles (thirty-two loads in flight) with
+// clamped addresses and masked values, straight-line code per batch.
+template <int STEP>
+__device__ __forceinline__ void splitk_column_pair_run(const float* __restrict__ partials, size_t tstride,
+                                                       unsigned col, int t_begin, int ktiles, float* a, float* b) {
+    constexpr int TB = 16;
+    float sa = *a, sb = *b;
+    for (int t0 = t_begin; t0 < ktiles; t0 += STEP * TB) {
+        float va[TB], vb[TB];
+#pragma unroll
+        for (int u = 0; u < TB; u++) {
+            const int t = t0 + STEP * u;
+            const int tc = t < ktiles ? t : ktiles - 1;
+            const float* src = partials + static_cast<size_t>(tc) * tstride + col;
+            const float ga = load_agent(src);
+            const float gb = load_agent(src + kWave);
+            va[u] = t < ktiles ? ga : 0.0f;
+            vb[u] = t < ktiles ? gb : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < TB; u++) {
+            sa += va[u];
+            sb += vb[u];
+        }
+    }
+    *a = sa;
+    *b = sb;
+}
+
+// One activation row, more than one K tile, and an epilogue that works on heads of 128 columns (two waves of
+// the tile): the two waves of a head share an arrival counter (lines kCountersPerTile * tile + 2 * (head in
+// tile)), every wave reports for itself as in splitk_exchange_sum_per_wave, and the last of the head's
+// 2 * ktiles waves reads both halves back: lane i ends up with columns i (`lo`) and i + 64 (`hi`) of the
+// head, the layout of the rotary routine.  Per column the additions run as in splitk_exchange_sum.
+// Returns true, the same in every lane, in that last wave; every other wave returns false and is done.
+// N is a multiple of 256 here (whole tiles of two heads).
+__device__ __forceinline__ bool splitk_exchange_sum_per_head(float psum, float* lo, float* hi, int N, int ct, int kt,
+                                                             int ktiles, float* __restrict__ partials,
+                                                             uint32_t* __restrict__ counters) {
+    const int tid = threadIdx.x;
+    if (tid >= kTileCols) return false;  // whole waves: the others own no column
+    const int col = ct * kTileCols + tid;
+    const size_t tstride = static_cast<size_t>(N);
+    store_agent(partials + static_cast<size_t>(kt) * tstride + col, psum);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    const int head_in_tile = tid / (2 * kWave);
+    uint32_t* counter = counters + (static_cast<size_t>(ct) * kCountersPerTile + 2 * head_in_tile) * kCounterStride;
+    uint32_t prev = 0;
+    if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = __builtin_amdgcn_readfirstlane(prev);
+    if (prev != static_cast<uint32_t>(2 * ktiles - 1)) return false;
+
+    // last of its head: every other wave's partial sums were acknowledged before its increment
+    const int first = ct * kTileCols + head_in_tile * 2 * kWave + tid % kWave;
+    float a = 0.0f, b = 0.0f;
+    if (!(ktiles > 16 && blockDim.x >= 2 * kTileCols)) {
+        splitk_column_pair_run<1>(partials, tstride, static_cast<unsigned>(first), 0, ktiles, &a, &b);
+    } else {
+        // where splitk_exchange_sum has helper threads: the even tiles in order, the odd ones likewise, even + odd
+        float ao = 0.0f, bo = 0.0f;
+        splitk_column_pair_run<2>(partials, tstride, static_cast<unsigned>(first), 0, ktiles, &a, &b);
+        splitk_column_pair_run<2>(partials, tstride, static_cast<unsigned>(first), 1, ktiles, &ao, &bo);
+        a += ao;
+        b += bo;
+    }
+    *lo = a;
+    *hi = b;
+    if (tid % kWave == 0) {
+        // leave the workspace ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+
 // The exchange for several activation rows (ROWS = 4, 8 or 16) and a workgroup of exactly 256 threads, more
 // than one K tile.  Partial sums go out as above, one column per thread.  The last workgroup reads them back
 // two columns per load: threads 0..127 take rows 0 .. ROWS/2-1 of column pairs 0..127, threads 128..255 the
