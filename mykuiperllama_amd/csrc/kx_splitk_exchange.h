@@ -48,6 +48,21 @@ __device__ __forceinline__ float load_agent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The partial sums as a buffer for the read-backs that use buffer loads: the lane's column is one vector
+// register shared by every load, a K tile's offset (the same in every lane) a scalar register, so that a load
+// costs one instruction and no address arithmetic in the vector unit.  The host keeps the partial sums below
+// 4 GiB.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t partials_buffer(float* partials, size_t floats) {
+    return __builtin_amdgcn_make_buffer_rsrc(partials, 0, static_cast<int>(static_cast<uint32_t>(floats * sizeof(float))),
+                                             0x00020000);
+}
+// Element `lane_bytes / 4` of the K tile that starts `tile_floats` floats into the buffer, device scope (cache
+// policy 16 is the sc1 bit, what load_agent's loads carry).
+__device__ __forceinline__ float load_partial(__amdgpu_buffer_rsrc_t rsrc, int lane_bytes, uint32_t tile_floats) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes,
+                                                                          static_cast<int>(tile_floats * 4u), 16));
+}
+
 // Called by every thread of the workgroup (it contains barriers).  Thread tid < 256 owns tile column
 // tid and brings psum[r], its partial sum for activation row m0 + r.  `s_prev` is one uint32 of LDS.
 // Returns true, the same in every thread, in the workgroup that ends up with the finished sums
@@ -199,7 +214,9 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_wave(float psum, float* 
 
     // last of its quarter: every other wave's partial sums were acknowledged before its increment
     constexpr int TB = 16;
-    const unsigned hcol = static_cast<unsigned>(col_ok ? col : N - 1);
+    const int lane_bytes = (col_ok ? col : N - 1) * static_cast<int>(sizeof(float));
+    const __amdgpu_buffer_rsrc_t rsrc = partials_buffer(partials, static_cast<size_t>(ktiles) * tstride);
+    const uint32_t tfloats = static_cast<uint32_t>(N);  // floats between consecutive K tiles
     float sum = 0.0f;
     if (!(ktiles > TB && blockDim.x >= 2 * kTileCols)) {
         for (int t0 = 0; t0 < ktiles; t0 += TB) {
@@ -209,38 +226,37 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_wave(float psum, float* 
                 // clamped address, masked value: the loads of a batch are straight-line code
                 const int t = t0 + u;
                 const int tc = t < ktiles ? t : ktiles - 1;
-                const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
+                const float got = load_partial(rsrc, lane_bytes, static_cast<uint32_t>(tc) * tfloats);
                 v[u] = t < ktiles ? got : 0.0f;
             }
 #pragma unroll
             for (int u = 0; u < TB; u++) sum += v[u];
         }
     } else {
-        // where splitk_exchange_sum has helper threads: the even tiles in order, the odd ones likewise, even + odd
+        // where splitk_exchange_sum has helper threads: the even tiles in order, the odd ones likewise, even + odd.
+        // Both runs are in flight together (thirty-two loads per batch).
         float odd = 0.0f;
         for (int t0 = 0; t0 < ktiles; t0 += 2 * TB) {
-            float v[TB];
+            // the even run is requested first: its additions start while the odd run is still arriving
+            float ve[TB], vo[TB];
 #pragma unroll
             for (int u = 0; u < TB; u++) {
                 const int t = t0 + 2 * u;
                 const int tc = t < ktiles ? t : ktiles - 1;
-                const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
-                v[u] = t < ktiles ? got : 0.0f;
+                const float got = load_partial(rsrc, lane_bytes, static_cast<uint32_t>(tc) * tfloats);
+                ve[u] = t < ktiles ? got : 0.0f;
             }
-#pragma unroll
-            for (int u = 0; u < TB; u++) sum += v[u];
-        }
-        for (int t0 = 1; t0 < ktiles; t0 += 2 * TB) {
-            float v[TB];
 #pragma unroll
             for (int u = 0; u < TB; u++) {
-                const int t = t0 + 2 * u;
+                const int t = t0 + 2 * u + 1;
                 const int tc = t < ktiles ? t : ktiles - 1;
-                const float got = load_agent(partials + static_cast<size_t>(tc) * tstride + hcol);
-                v[u] = t < ktiles ? got : 0.0f;
+                const float got = load_partial(rsrc, lane_bytes, static_cast<uint32_t>(tc) * tfloats);
+                vo[u] = t < ktiles ? got : 0.0f;
             }
 #pragma unroll
-            for (int u = 0; u < TB; u++) odd += v[u];
+            for (int u = 0; u < TB; u++) sum += ve[u];
+#pragma unroll
+            for (int u = 0; u < TB; u++) odd += vo[u];
         }
         sum += odd;
     }
@@ -267,7 +283,7 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
 // `ktiles`, added to `a` and `b` in that order; batches of sixteen K tiles (thirty-two loads in flight) with
 // clamped addresses and masked values, straight-line code per batch.
 template <int STEP>
-__device__ __forceinline__ void splitk_column_pair_run(const float* __restrict__ partials, size_t tstride,
+__device__ __forceinline__ void splitk_column_pair_run(__amdgpu_buffer_rsrc_t rsrc, uint32_t tfloats,
                                                        unsigned col, int t_begin, int ktiles, float* a, float* b) {
     constexpr int TB = 16;
     float sa = *a, sb = *b;
@@ -277,9 +293,8 @@ __device__ __forceinline__ void splitk_column_pair_run(const float* __restrict__
         for (int u = 0; u < TB; u++) {
             const int t = t0 + STEP * u;
             const int tc = t < ktiles ? t : ktiles - 1;
-            const float* src = partials + static_cast<size_t>(tc) * tstride + col;
-            const float ga = load_agent(src);
-            const float gb = load_agent(src + kWave);
+            const float ga = load_partial(rsrc, static_cast<int>(col * sizeof(float)), static_cast<uint32_t>(tc) * tfloats);
+            const float gb = load_partial(rsrc, static_cast<int>((col + kWave) * sizeof(float)), static_cast<uint32_t>(tc) * tfloats);
             va[u] = t < ktiles ? ga : 0.0f;
             vb[u] = t < ktiles ? gb : 0.0f;
         }
@@ -319,14 +334,16 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_head(float psum, float* 
 
     // last of its head: every other wave's partial sums were acknowledged before its increment
     const int first = ct * kTileCols + head_in_tile * 2 * kWave + tid % kWave;
+    const __amdgpu_buffer_rsrc_t rsrc = partials_buffer(partials, static_cast<size_t>(ktiles) * tstride);
+    const uint32_t tfloats = static_cast<uint32_t>(N);  // floats between consecutive K tiles
     float a = 0.0f, b = 0.0f;
     if (!(ktiles > 16 && blockDim.x >= 2 * kTileCols)) {
-        splitk_column_pair_run<1>(partials, tstride, static_cast<unsigned>(first), 0, ktiles, &a, &b);
+        splitk_column_pair_run<1>(rsrc, tfloats, static_cast<unsigned>(first), 0, ktiles, &a, &b);
     } else {
         // where splitk_exchange_sum has helper threads: the even tiles in order, the odd ones likewise, even + odd
         float ao = 0.0f, bo = 0.0f;
-        splitk_column_pair_run<2>(partials, tstride, static_cast<unsigned>(first), 0, ktiles, &a, &b);
-        splitk_column_pair_run<2>(partials, tstride, static_cast<unsigned>(first), 1, ktiles, &ao, &bo);
+        splitk_column_pair_run<2>(rsrc, tfloats, static_cast<unsigned>(first), 0, ktiles, &a, &b);
+        splitk_column_pair_run<2>(rsrc, tfloats, static_cast<unsigned>(first), 1, ktiles, &ao, &bo);
         a += ao;
         b += bo;
     }
