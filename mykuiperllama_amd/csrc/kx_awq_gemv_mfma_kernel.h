@@ -415,9 +415,12 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < ROWS; r++) sum[r] = s_sum[r * kTileCols + tid];
             }
+        } else if constexpr (EPI == kEpiResidual) {
+            // every wave of 64 columns finishes for itself: the epilogue below needs nothing from the other waves
+            load_residual();
+            if (!splitk_exchange_sum_per_wave_rows<ROWS>(psum, sum, M, N, ct, kt, ktiles, partials, counters)) return;
         } else {
             if (!splitk_exchange_sum<ROWS>(psum, sum, 0, M, N, ct, kt, ktiles, ct, partials, counters, &s_prev)) return;
-            load_residual();
         }
         if constexpr (EPI == kEpiQkRope) {
             // The finished rows, rounded to bf16 as a separate GEMV would store them, go through LDS so that a
@@ -462,7 +465,15 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         static_assert(THREADS == kTileCols, "the wide exchange is laid out for 256 threads");
         splitk_exchange_store_wide<ROWS>(psum, M, N, ct, kt, ktiles, partials, counters, y, &s_prev);
     } else {
-        splitk_exchange_store<ROWS>(psum, 0, M, N, ct, kt, ktiles, ct, partials, counters, y, &s_prev);
+        // one or two activation rows: every wave of 64 columns is an exchange of its own
+        float sum[ROWS];
+        if (!splitk_exchange_sum_per_wave_rows<ROWS>(psum, sum, M, N, ct, kt, ktiles, partials, counters)) return;
+        if (own_col < N) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (r < M) y[static_cast<size_t>(r) * N + own_col] = f32_to_bf16(sum[r]);
+            }
+        }
     }
 }
 

@@ -279,6 +279,77 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
     if (col < N) y[col] = f32_to_bf16(sum);
 }
 
+// The per-wave exchange for ROWS activation rows (M <= ROWS of them live) of a workgroup of 256 threads:
+// partial sums laid out [K tile][M][N] as in splitk_exchange_sum, one arrival counter per wave of 64 columns,
+// the last wave of a quarter reads every row of its columns back, K tiles in order (the order of
+// splitk_exchange_sum without helper threads, so the bits are those of that routine).
+// Returns true, the same in every lane, in the wave that ends up with the finished sums (`sum`, rows at or
+// past M are zero); the other waves return false and are done.
+template <int ROWS>
+__device__ __forceinline__ bool splitk_exchange_sum_per_wave_rows(const float (&psum)[ROWS], float (&sum)[ROWS], int M,
+                                                                  int N, int ct, int kt, int ktiles,
+                                                                  float* __restrict__ partials,
+                                                                  uint32_t* __restrict__ counters) {
+    static_assert(ROWS >= 1 && ROWS <= 4, "sixteen K tiles of every row are in flight together");
+    const int tid = threadIdx.x;
+    if (tid >= kTileCols) return false;  // whole waves: the others own no column
+    if (ktiles == 1) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) sum[r] = r < M ? psum[r] : 0.0f;
+        return true;
+    }
+    const int col = ct * kTileCols + tid;
+    const bool col_ok = col < N;
+    const size_t tstride = static_cast<size_t>(M) * N;  // floats between consecutive K tiles
+    if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            if (r < M) store_agent(partials + static_cast<size_t>(kt) * tstride + static_cast<size_t>(r) * N + col, psum[r]);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    uint32_t* counter = counters + (static_cast<size_t>(ct) * kCountersPerTile + tid / kWave) * kCounterStride;
+    uint32_t prev = 0;
+    if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    prev = __builtin_amdgcn_readfirstlane(prev);
+    if (prev != static_cast<uint32_t>(ktiles - 1)) return false;
+
+    // last of its quarter: every other wave's partial sums were acknowledged before its increment
+    constexpr int TB = 16;
+    const int lane_bytes = (col_ok ? col : N - 1) * static_cast<int>(sizeof(float));
+    const __amdgpu_buffer_rsrc_t rsrc = partials_buffer(partials, static_cast<size_t>(ktiles) * tstride);
+    const uint32_t tfloats = static_cast<uint32_t>(tstride);
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) sum[r] = 0.0f;
+    for (int t0 = 0; t0 < ktiles; t0 += TB) {
+        float v[ROWS][TB];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+#pragma unroll
+            for (int u = 0; u < TB; u++) {
+                // clamped address, masked value: the loads of a batch are straight-line code
+                const int t = t0 + u;
+                const int tc = t < ktiles ? t : ktiles - 1;
+                const int rc = r < M ? r : M - 1;
+                const float got = load_partial(rsrc, lane_bytes, static_cast<uint32_t>(tc) * tfloats +
+                                                                     static_cast<uint32_t>(rc) * static_cast<uint32_t>(N));
+                v[r][u] = (t < ktiles && r < M) ? got : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+#pragma unroll
+            for (int u = 0; u < TB; u++) sum[r] += v[r][u];
+        }
+    }
+    if (tid % kWave == 0) {
+        // leave the workspace ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+
 // Sums of the partial sums of columns `col` and `col + 64` over K tiles t_begin, t_begin + STEP, ... below
 // `ktiles`, added to `a` and `b` in that order; batches of sixteen K tiles (thirty-two loads in flight) with
 // clamped addresses and masked values, straight-line code per batch.
