@@ -9,7 +9,8 @@
 
 `python -m mykuiperllama_amd.build --ablate N` additionally builds lib/libkx_hip_ablateN.so, the HIP
 library with parts of the GEMV kernels compiled out (-DKX_ABLATE=N: 1 = no split-K exchange, 2 = loads
-only); `bench.py --lib` times it.  Its results are wrong by construction: it exists to attribute time.
+only, 3 = loads and arithmetic but neither the reduction across lanes and waves nor the exchange, on the
+vector kernel's plain launch; the other kernels as with 1); `bench.py --lib` times it.  Its results are wrong by construction: it exists to attribute time.
 
 Everything lands under mykuiperllama_amd/lib/, in-tree, so that a snapshot of the repository
 carries the binaries to a machine that only runs them.

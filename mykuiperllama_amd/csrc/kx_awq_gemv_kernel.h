@@ -291,7 +291,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         // keep the scheduler from sinking loads below the first use of an earlier one
         __builtin_amdgcn_sched_barrier(0);
     }
-#if defined(KX_ABLATE) && KX_ABLATE >= 2
+#if defined(KX_ABLATE) && KX_ABLATE == 2
     if constexpr (!STAGED) {
         if (ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
             uint32_t f = zw ^ sraw.x ^ sraw.y ^ sraw.z ^ sraw.w;
@@ -475,6 +475,20 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
     }
 
+#if defined(KX_ABLATE) && KX_ABLATE == 3
+    if constexpr (!STAGED) {
+        if (ktiles > 1) {  // profiling build: loads and arithmetic - no reduction across lanes and waves, no exchange
+            float f = 0.0f;
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+#pragma unroll
+                for (int c = 0; c < 8; c++) f += acc[m][c];
+            }
+            if (f == 12345.678f) partials[tid] = 1.0f;
+            return;
+        }
+    }
+#endif
     // The two row slots of a wave meet through a lane exchange, the waves of the workgroup in
     // LDS (one activation row at a time); afterwards thread t < 256 owns tile column t.
     static_assert(kSlotsPerWave == 2, "the lane exchange below pairs lane l with lane l + 32");

@@ -222,7 +222,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         }
     }
     __builtin_amdgcn_sched_barrier(0);
-#if defined(KX_ABLATE) && KX_ABLATE >= 2
+#if defined(KX_ABLATE) && KX_ABLATE == 2
     if (!STAGED && ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
         uint32_t f = 0;
 #pragma unroll
