@@ -226,6 +226,41 @@ def test_norm_input_with_rotary_output(capi, torch):
         assert rel_l2(a, b) <= 5e-3
 
 
+@pytest.mark.parametrize("K", [8192, 12288])
+def test_row_input_with_rotary_output_on_tall_k(capi, torch, K):
+    """32 and 48 K tiles per column: the finishing wave of a head adds the even and the odd tiles separately, in one
+    and in two batches of each, and must return the bits of the plain launch followed by the per-head kernel."""
+    n_q, n_kv, group, eps, theta, pos_value, max_pos = 2, 1, 128, 1e-6, 1e6, 5, 8
+    N = (n_q + 2 * n_kv) * 128
+    qw, sc, qz = weights(torch, f"chain_rope_tall_{K}", K, N, group)
+    x = bf16_rand(torch, (1, K), K)
+    hg = (1 + 0.1 * torch.randn((128,), device="cuda")).bfloat16()
+    pos = torch.tensor([pos_value], dtype=torch.int32, device="cuda")
+    ws = capi.make_workspace(1, K, N)
+    qkv = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_bf16(x, qw, sc, qz, qkv, group, ws)
+    q_sep = torch.empty((1, n_q * 128), dtype=torch.bfloat16, device="cuda")
+    k_sep = torch.zeros((max_pos, n_kv, 128), dtype=torch.bfloat16, device="cuda")
+    v_sep = torch.zeros_like(k_sep)
+    capi.qk_norm_rope_bf16(qkv, hg, hg, q_sep, k_sep, v_sep, n_q, n_kv, pos, theta, eps)
+
+    for _ in range(2):  # the second launch finds the counters as the first one left them
+        q_one = torch.full_like(q_sep, float("nan"))
+        k_one, v_one = torch.zeros_like(k_sep), torch.zeros_like(v_sep)
+        capi.gemv_awq_chain_bf16({"in_kind": capi.IN_ROW, "x": x, "out_kind": capi.OUT_QKV_ROPE, "q_gain": hg,
+                                  "k_gain": hg, "q_out": q_one, "k_cache": k_one, "v_cache": v_one, "pos": pos,
+                                  "rope_n_q_heads": n_q, "rope_n_kv_heads": n_kv, "rope_theta": theta, "qk_eps": eps},
+                                 qw, sc, qz, K, N, group, ws)
+        torch.cuda.synchronize()
+        for a, b in ((q_one, q_sep), (k_one, k_sep), (v_one, v_sep)):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # and the plain launch still works on the same workspace
+    again = torch.empty_like(qkv)
+    capi.gemv_awq_bf16(x, qw, sc, qz, again, group, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(again.view(torch.int16), qkv.view(torch.int16))
+
+
 def test_chain_rejects_bad_descriptors(capi, torch):
     K, N, group = 512, 512, 128
     qw, sc, qz = weights(torch, "chain_bad", K, N, group)

@@ -166,6 +166,7 @@ QKV_CASES = [
     (512, 4, 2, 128, True),
     (128, 2, 1, 32, True),       # four waves per workgroup
     (64, 2, 2, 32, True),        # K in one workgroup: no split, every workgroup finishes its own tile
+    (8192, 4, 2, 128, True),     # 32 K tiles: the read-back adds the even and the odd tiles separately
 ]
 
 
