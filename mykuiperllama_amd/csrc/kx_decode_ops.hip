@@ -268,8 +268,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         }
         l = wave_sum(l);
         if (lane == 0) {
-            ml_base[2 * g] = m;
-            ml_base[2 * g + 1] = l;
+            store_result(ml_base + 2 * g, m);
+            store_result(ml_base + 2 * g + 1, l);
         }
     }
     // The V rows go to LDS while the statistics are being taken: rows past the context carry weight 0,
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int head = 4 * mb + v;
-            if (head < G) out_base[head * kHeadDim + col] = dacc[n][v];
+            if (head < G) store_result(out_base + head * kHeadDim + col, dacc[n][v]);
         }
     }
 }

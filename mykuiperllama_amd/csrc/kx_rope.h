@@ -60,8 +60,8 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     if (head >= t.n_q + t.n_kv) {  // value head: straight into the cache
         if (row_ok) {
             uint16_t* dst = t.v_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q - t.n_kv)) * kHeadDim;
-            dst[lane] = a_bits;
-            dst[lane + 64] = b_bits;
+            store_result(dst + lane, a_bits);
+            store_result(dst + lane + 64, b_bits);
         }
         return;
     }
@@ -83,12 +83,12 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     // two guarded stores rather than one store through a selected pointer (see qk_norm_rope_head)
     if (is_q) {
         uint16_t* dst = t.q_out + static_cast<size_t>(head) * kHeadDim;
-        dst[lane] = f32_to_bf16(oa);
-        dst[lane + 64] = f32_to_bf16(ob);
+        store_result(dst + lane, f32_to_bf16(oa));
+        store_result(dst + lane + 64, f32_to_bf16(ob));
     } else if (row_ok) {
         uint16_t* dst = t.k_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q)) * kHeadDim;
-        dst[lane] = f32_to_bf16(oa);
-        dst[lane + 64] = f32_to_bf16(ob);
+        store_result(dst + lane, f32_to_bf16(oa));
+        store_result(dst + lane + 64, f32_to_bf16(ob));
     }
 }
 
