@@ -560,7 +560,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             if (tid < kTileCols && (tid & 64) == 0) {
                 const int local = tid >> 7;
                 const int head = ct * (kTileCols / kHeadDim) + local;
-                qk_norm_rope_head_with(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane,
+                qk_norm_rope_head_with<true>(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane,
                                        rope, rope_pos, rope_gain_a, rope_gain_b);
             }
         } else {
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             float lo, hi;
             if (!splitk_exchange_sum_per_head(psum[0], &lo, &hi, N, ct, kt, ktiles, partials, counters)) return;
             const int head = ct * (kTileCols / kHeadDim) + (tid >> 7);
-            qk_norm_rope_head_with(f32_to_bf16(lo), f32_to_bf16(hi), head, lane, rope, rope_pos, rope_gain_a,
+            qk_norm_rope_head_with<true>(f32_to_bf16(lo), f32_to_bf16(hi), head, lane, rope, rope_pos, rope_gain_a,
                                    rope_gain_b);
         }
     }

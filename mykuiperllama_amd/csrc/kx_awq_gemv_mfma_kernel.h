@@ -452,12 +452,12 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
                 if (col_ok && r < M) {
                     const float o = bf16_to_f32(f32_to_bf16(sum[r]));  // the projection's output is a bf16 tensor
                     const uint16_t rbits = f32_to_bf16(bf16_to_f32(rin[r]) + o);
-                    store_result(res.out + static_cast<size_t>(r) * N + own_col, rbits);
+                    res.out[static_cast<size_t>(r) * N + own_col] = rbits;
                     rv = bf16_to_f32(rbits);
                 }
                 const float q = wave_sum(rv * rv);
                 if (lane == 0 && r < M) {
-                    store_result(res.sumsq + (static_cast<size_t>(r) * gridDim.x + ct) * (kTileCols / kWave) + wave, q);
+                    res.sumsq[(static_cast<size_t>(r) * gridDim.x + ct) * (kTileCols / kWave) + wave] = q;
                 }
             }
         }
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         if (own_col < N) {
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
-                if (r < M) store_result(y + static_cast<size_t>(r) * N + own_col, f32_to_bf16(sum[r]));
+                if (r < M) y[static_cast<size_t>(r) * N + own_col] = f32_to_bf16(sum[r]);
             }
         }
     }

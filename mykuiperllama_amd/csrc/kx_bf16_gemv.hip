@@ -91,7 +91,9 @@ __global__ __launch_bounds__(kRowsPerBlock * kWave) void bf16_gemv_kernel(
     if (lane == 0 && n < N) {
 #pragma unroll
         for (int m = 0; m < MB; m++) {
-            if (m0 + m < M) store_result(y + static_cast<size_t>(m0 + m) * N + n, f32_to_bf16(acc[m]));
+            // a plain store: one wave owns one column, and two-byte write-through stores from 150 000 waves cost
+            // the lm_head launch 8 us
+            if (m0 + m < M) y[static_cast<size_t>(m0 + m) * N + n] = f32_to_bf16(acc[m]);
         }
     }
 }
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(kMfmaWaves * kWave) void bf16_gemv_mfma_kernel(
         for (int v = 0; v < 4; v++) {
             const int m = 4 * b + v;
             const float sum = (red[0][wave][v][lane] + red[1][wave][v][lane]) + (red[2][wave][v][lane] + red[3][wave][v][lane]);
-            if (m < M) store_result(y + static_cast<size_t>(m) * N + n, f32_to_bf16(sum));
+            if (m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16(sum);
         }
     }
 }

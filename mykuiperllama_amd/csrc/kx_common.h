@@ -58,9 +58,11 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return static_cast<float>(v);
 }
 
-// A kernel's results leave with the device-scope bit: the store is written through the XCD's L2 to memory at
-// once, so the end of the kernel finds no dirty lines to write back.  Measured on the one-row AWQ GEMV:
-// 0.1-0.2 us per launch (1.9 % on the seven-projection step) against plain stores.
+// The results of a one-row launch leave with the device-scope bit: the store is written through the XCD's L2 to
+// memory at once, so the end of the kernel finds no dirty lines to write back.  Measured on the one-row AWQ
+// GEMV: 0.1-0.2 us per launch (1.9 % on the seven-projection step) against plain stores.  Not for bulk: the
+// launches of a step with 8 or 16 sequences write enough for the write-through traffic to cost 1.5-4 % of the
+// step, and 150 000 waves that each store two bytes of an lm_head row lose 8 us; those keep plain stores.
 template <typename T>
 __device__ __forceinline__ void store_result(T* p, T v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -217,6 +217,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     const int ctx = pos_ptr[0] + 1;  // positions 0 .. pos are valid (pos was appended just before)
     __builtin_amdgcn_sched_barrier(0);
 
+    const bool one_sequence = gridDim.z == 1;  // write-through results for the one-row step only (store_result)
     float* out_base = part_out + (static_cast<size_t>(kvh) * nchunks + chunk) * G * kHeadDim;
     float* ml_base = part_ml + (static_cast<size_t>(kvh) * nchunks + chunk) * G * 2;
     // No early exit for a chunk past the end of the context: a branch on *pos ahead of the loads
@@ -268,8 +269,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         }
         l = wave_sum(l);
         if (lane == 0) {
-            store_result(ml_base + 2 * g, m);
-            store_result(ml_base + 2 * g + 1, l);
+            if (one_sequence) {
+                store_result(ml_base + 2 * g, m);
+                store_result(ml_base + 2 * g + 1, l);
+            } else {
+                ml_base[2 * g] = m;
+                ml_base[2 * g + 1] = l;
+            }
         }
     }
     // The V rows go to LDS while the statistics are being taken: rows past the context carry weight 0,
@@ -335,7 +341,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int head = 4 * mb + v;
-            if (head < G) store_result(out_base + head * kHeadDim + col, dacc[n][v]);
+            if (head < G) {
+                if (one_sequence) store_result(out_base + head * kHeadDim + col, dacc[n][v]);
+                else out_base[head * kHeadDim + col] = dacc[n][v];
+            }
         }
     }
 }

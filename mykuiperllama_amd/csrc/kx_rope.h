@@ -45,6 +45,13 @@ __device__ __forceinline__ void rope_sincos(float x, float* s_out, float* c_out)
     *c_out = ((q + 1) & 2) ? -ca : ca;
 }
 
+// The routine's stores: write-through (store_result) for the one-row launch that ends with them, plain otherwise.
+template <bool WRITE_THROUGH>
+__device__ __forceinline__ void rope_store(uint16_t* p, uint16_t v) {
+    if constexpr (WRITE_THROUGH) store_result(p, v);
+    else *p = v;
+}
+
 // Called by the 64 lanes of one wave; lane i brings elements i and i + 64 of head `head`
 // (0 .. n_q + 2 n_kv - 1, query heads first, then key heads, then value heads) as bf16 bits.
 //   out[i]      = x[i] * cos(pos f_i) - x[i+64] * sin(pos f_i)
@@ -53,6 +60,7 @@ __device__ __forceinline__ void rope_sincos(float x, float* s_out, float* c_out)
 // `pos`, `gain_a` and `gain_b` are *t.pos and elements lane and lane + 64 of the head's gain (q_gain for a
 // query head, k_gain for a key head, unused for a value head): a caller that knows early which head
 // a wave will serve loads them ahead of time.
+template <bool WRITE_THROUGH = false>
 __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t b_bits, int head, int lane,
                                                        const RopeTarget& t, int pos, uint16_t gain_a,
                                                        uint16_t gain_b) {
@@ -60,8 +68,8 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     if (head >= t.n_q + t.n_kv) {  // value head: straight into the cache
         if (row_ok) {
             uint16_t* dst = t.v_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q - t.n_kv)) * kHeadDim;
-            store_result(dst + lane, a_bits);
-            store_result(dst + lane + 64, b_bits);
+            rope_store<WRITE_THROUGH>(dst + lane, a_bits);
+            rope_store<WRITE_THROUGH>(dst + lane + 64, b_bits);
         }
         return;
     }
@@ -83,12 +91,12 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     // two guarded stores rather than one store through a selected pointer (see qk_norm_rope_head)
     if (is_q) {
         uint16_t* dst = t.q_out + static_cast<size_t>(head) * kHeadDim;
-        store_result(dst + lane, f32_to_bf16(oa));
-        store_result(dst + lane + 64, f32_to_bf16(ob));
+        rope_store<WRITE_THROUGH>(dst + lane, f32_to_bf16(oa));
+        rope_store<WRITE_THROUGH>(dst + lane + 64, f32_to_bf16(ob));
     } else if (row_ok) {
         uint16_t* dst = t.k_cache + (static_cast<size_t>(pos) * t.n_kv + (head - t.n_q)) * kHeadDim;
-        store_result(dst + lane, f32_to_bf16(oa));
-        store_result(dst + lane + 64, f32_to_bf16(ob));
+        rope_store<WRITE_THROUGH>(dst + lane, f32_to_bf16(oa));
+        rope_store<WRITE_THROUGH>(dst + lane + 64, f32_to_bf16(ob));
     }
 }
 

@@ -169,7 +169,7 @@ __device__ __forceinline__ void splitk_exchange_store(const float (&psum)[ROWS],
     if (threadIdx.x < kTileCols && col < N) {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
-            if (m0 + r < M) store_result(y + static_cast<size_t>(m0 + r) * N + col, f32_to_bf16(sum[r]));
+            if (m0 + r < M) y[static_cast<size_t>(m0 + r) * N + col] = f32_to_bf16(sum[r]);
         }
     }
 }
@@ -530,7 +530,7 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
         if (col < N) {
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
-                if (r < M) store_result(y + static_cast<size_t>(r) * N + col, f32_to_bf16(psum[r]));
+                if (r < M) y[static_cast<size_t>(r) * N + col] = f32_to_bf16(psum[r]);
             }
         }
         return;
@@ -545,7 +545,7 @@ __device__ __forceinline__ void splitk_exchange_store_wide(const float (&psum)[R
         for (int i = 0; i < HALF; i++) {
             const int m = row0 + i;
             if (m < M) {
-                store_result(reinterpret_cast<uint32_t*>(y + static_cast<size_t>(m) * N + col2), f32x2_to_bf16x2(lo[i], hi[i]));
+                *reinterpret_cast<uint32_t*>(y + static_cast<size_t>(m) * N + col2) = f32x2_to_bf16x2(lo[i], hi[i]);
             }
         }
     }
