@@ -10,8 +10,8 @@
 //   y_part[n] = s[g,n] * ( sum_r (16 + q[k0+r,n]) * x[k0+r]  -  (16 + z[g,n]) * sum_r x[k0+r] )
 //
 // A wave covers 32 consecutive word columns (128 contiguous bytes of each row, 256 output
-// columns) times two row slots; a workgroup stacks WAVES waves along K.  The two row slots of a
-// wave meet through a lane exchange, the waves of a workgroup in LDS.
+// columns) times two row slots; a workgroup stacks WAVES waves along K.  All row slots of a
+// workgroup meet in LDS.
 // Workgroups that share a column tile meet in a caller-provided workspace: each stores its 256
 // partial sums, then bumps the tile's arrival counter; the workgroup that arrives last adds the
 // partials in a fixed order (bitwise reproducible) and writes y.  Thread t of a workgroup owns
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     static_assert(RT % 8 == 0, "a lane reads its activations in 16-byte pieces");
     static_assert(KB <= THREADS, "one staging thread per row of the workgroup's K range");
 
-    __shared__ __attribute__((aligned(16))) float red[WAVES][kTileCols];
+    __shared__ __attribute__((aligned(16))) float red[WAVES * kSlotsPerWave][kTileCols];
     __shared__ __attribute__((aligned(16))) uint16_t s_x[STAGED ? MB : 1][STAGED ? KB : 8];  // staged activations, bf16
     __shared__ float s_ss[NORM ? MB : 1][WAVES];
     __shared__ __attribute__((aligned(16))) float s_factor[MERGE ? HB : 1][MERGE ? kMergeParts * kMergeHold : 4];
@@ -489,31 +489,32 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
     }
 #endif
-    // The two row slots of a wave meet through a lane exchange, the waves of the workgroup in
-    // LDS (one activation row at a time); afterwards thread t < 256 owns tile column t.
-    static_assert(kSlotsPerWave == 2, "the lane exchange below pairs lane l with lane l + 32");
+    // The row slots of the workgroup meet in LDS (one activation row at a time); afterwards thread t < 256 owns
+    // tile column t.  (A lane exchange between the two slots of a wave in front of the LDS round — a shuffle by
+    // 32 lanes, itself an LDS round trip — halved the LDS traffic and cost 0.1 us per launch.)
+    static_assert(kSlotsPerWave == 2, "the sum below pairs the two row slots of a wave");
     static_assert(WAVES * kWave >= kTileCols, "one thread per tile column");
     const int wave = tid / kWave;
     const int lane = tid % kWave;
     float psum[MB];
 #pragma unroll
     for (int m = 0; m < MB; m++) {
-#pragma unroll
-        for (int c = 0; c < 8; c++) acc[m][c] += __shfl_xor(acc[m][c], 32, kWave);
+        // every row slot leaves its eight sums in LDS; the two slots of a wave are added first, then the waves in
+        // order (the grouping a lane exchange inside the wave followed by a sum over the waves would give)
         if (m > 0) __syncthreads();  // the previous row has been read
-        if (lane < kWC) {
-            f32x4* dst = reinterpret_cast<f32x4*>(&red[wave][8 * lane]);
+        {
+            f32x4* dst = reinterpret_cast<f32x4*>(&red[slot][8 * wc]);
             dst[0] = f32x4{acc[m][0], acc[m][1], acc[m][2], acc[m][3]};
             dst[1] = f32x4{acc[m][4], acc[m][5], acc[m][6], acc[m][7]};
         }
         __syncthreads();
         psum[m] = 0.0f;
         if (tid < kTileCols) {
-            float v[WAVES];
+            float v[SLOTS];
 #pragma unroll
-            for (int u = 0; u < WAVES; u++) v[u] = red[u][tid];
+            for (int u = 0; u < SLOTS; u++) v[u] = red[u][tid];
 #pragma unroll
-            for (int u = 0; u < WAVES; u++) psum[m] += v[u];
+            for (int u = 0; u < WAVES; u++) psum[m] += v[2 * u] + v[2 * u + 1];
         }
     }
 
