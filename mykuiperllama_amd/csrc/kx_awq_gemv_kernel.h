@@ -428,6 +428,24 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         float xsum[MB];
 #pragma unroll
         for (int m = 0; m < MB; m++) xsum[m] = 0.0f;
+        // Scale and 16 + zero point of the lane's eight columns: they arrived ahead of the weights, and what is
+        // converted here does not stand between the last weight row and the reduction.  With 32 rows per lane the
+        // sixteen registers this keeps across the loop cost more than the shorter tail gains (measured), and
+        // the conversion stays behind the loop.
+        constexpr bool kConvertEarly = RT <= 16;
+        float col_scale[8], col_zoff[8];
+        if constexpr (kConvertEarly) {
+            float z[8];
+            unpack_codes(zw, z);
+            const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
+                col_scale[c] = f16_bits_to_f32(bits);
+                col_zoff[c] = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
 #pragma unroll
         for (int rp = 0; rp < RT / 2; rp++) {
@@ -460,17 +478,22 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
 
         // zero point and scale, once per lane and column
-        float z[8];
-        unpack_codes(zw, z);
-        const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+        if constexpr (!kConvertEarly) {
+            float z[8];
+            unpack_codes(zw, z);
+            const uint32_t sw[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
+                col_scale[c] = f16_bits_to_f32(bits);
+                col_zoff[c] = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
+            }
+        }
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
-            const float sc = f16_bits_to_f32(bits);
-            const float zoff = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
 #pragma unroll
             for (int m = 0; m < MB; m++) {
-                acc[m][c] = sc * __builtin_fmaf(-zoff, xsum[m], acc[m][c]);
+                acc[m][c] = col_scale[c] * __builtin_fmaf(-col_zoff[c], xsum[m], acc[m][c]);
             }
         }
     }
