@@ -377,6 +377,14 @@ def main():
                                  "events on the launch stream; us = median per-launch time over the replays; "
                                  "stream_floor_us = the same for a kernel that only reads the shape's three packed "
                                  "tensors (mykuiperllama_amd/probe/kx_stream_probe.hip)"}
+        # what a launch costs before it has done anything: workgroups of 512 threads that return at once
+        def launch_empty(blocks):
+            def body(first, count):
+                for _ in range(count):
+                    capi.probe_empty_launch(blocks)
+            return body
+        per_shape["empty_launch_us"] = {str(b): spread(replay_times(torch, launch_empty(b), 60, 20))["us"]
+                                        for b in (64, 256, 768, 2000)}
         for n in ["k_proj", "q_proj", "gate_proj", "down_proj"]:
             K, N = shapes[n]
             per_shape[f"{n} {K}x{N}"] = shape_report(torch, capi, synth, K, N, group, [st.t[n] for st in sets],

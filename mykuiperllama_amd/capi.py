@@ -117,8 +117,7 @@ def load(path=None):
 _probe = None
 
 
-def probe_stream_read(buffers, sink=None):
-    """Measurement only: read up to three device tensors once with plain 16-byte loads (libkx_probe.so)."""
+def _load_probe():
     global _probe
     if _probe is None:
         import torch  # noqa: F401
@@ -128,6 +127,21 @@ def probe_stream_read(buffers, sink=None):
         _probe = ctypes.CDLL(PROBE_LIB)
         _probe.kx_probe_stream_read.restype = ctypes.c_int
         _probe.kx_probe_stream_read.argtypes = [_P, _SZ, _P, _SZ, _P, _SZ, _P, _P]
+        _probe.kx_probe_empty_launch.restype = ctypes.c_int
+        _probe.kx_probe_empty_launch.argtypes = [_I32, _P, _P]
+    return _probe
+
+
+def probe_empty_launch(blocks):
+    """Measurement only: a launch of `blocks` workgroups of 512 threads that do nothing (libkx_probe.so)."""
+    rc = _load_probe().kx_probe_empty_launch(blocks, None, _stream())
+    if rc != 0:
+        raise RuntimeError(f"kx_probe_empty_launch failed with HIP error {rc}")
+
+
+def probe_stream_read(buffers, sink=None):
+    """Measurement only: read up to three device tensors once with plain 16-byte loads (libkx_probe.so)."""
+    _load_probe()
     args = []
     for i in range(3):
         t = buffers[i] if i < len(buffers) else None

@@ -1,5 +1,5 @@
 // Measurement only (not part of the drop-in boundary): a kernel that reads given device buffers once with
-// plain 16-byte loads and does nothing else.  bench.py times it over the very tensors of a projection, with
+// plain 16-byte loads and does nothing else, and a kernel that does nothing at all.  bench.py times it over the very tensors of a projection, with
 // the same cold rotation and graph replay as the GEMV, and reports the result as the streaming floor of
 // that shape on this machine: what the memory system, the dispatcher and a kernel boundary cost when no
 // arithmetic, reduction or exchange is in the way.
@@ -39,7 +39,20 @@ __global__ __launch_bounds__(kThreads) void stream_read_kernel(Segments s, uint3
     if (fold == 0x9E3779B9u && sink) sink[0] = fold;  // keeps the loads alive; all but never taken
 }
 
+// A launch that does nothing: what the dispatcher and a kernel boundary cost on their own.
+__global__ __launch_bounds__(kThreads) void empty_kernel(uint32_t* sink) {
+    if (sink && blockIdx.x == 0xffffffffu) sink[0] = threadIdx.x;  // never taken
+}
+
 }  // namespace
+
+// Launches `blocks` workgroups of 512 threads that do nothing.  Returns 0 or a hipError_t.
+extern "C" int kx_probe_empty_launch(int blocks, void* sink, void* stream) {
+    if (blocks < 1) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(empty_kernel, dim3(blocks), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t*>(sink));
+    return static_cast<int>(hipGetLastError());
+}
 
 // Reads up to three device buffers (16-byte aligned, sizes rounded down to 16 bytes; a null or empty buffer is
 // skipped) once on `stream`.  `sink` is one writable device word, or null.  Returns 0 or a hipError_t.
