@@ -291,6 +291,13 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         // keep the scheduler from sinking loads below the first use of an earlier one
         __builtin_amdgcn_sched_barrier(0);
     }
+    // The rotation's sine and cosine while the weights are on their way: the vector unit has nothing to do yet,
+    // and the wave that finishes a head finds them ready instead of working them out behind the exchange.
+    float rope_sin = 0.0f, rope_cos = 1.0f;
+    if constexpr (EPI == kEpiQkRope) {
+        rope_angle(rope, rope_pos, tid % kWave, &rope_sin, &rope_cos);
+        __builtin_amdgcn_sched_barrier(0);
+    }
 #if defined(KX_ABLATE) && KX_ABLATE == 2
     if constexpr (!STAGED) {
         if (ktiles > 1) {  // profiling build: loads only - fold what arrived into one word and leave
@@ -584,16 +591,16 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             if (tid < kTileCols && (tid & 64) == 0) {
                 const int local = tid >> 7;
                 const int head = ct * (kTileCols / kHeadDim) + local;
-                qk_norm_rope_head_with<true>(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane,
-                                       rope, rope_pos, rope_gain_a, rope_gain_b);
+                qk_norm_rope_head_at<true>(s_row[local * kHeadDim + lane], s_row[local * kHeadDim + lane + 64], head, lane,
+                                           rope, rope_pos, rope_gain_a, rope_gain_b, rope_sin, rope_cos);
             }
         } else {
             // the last of the head's waves over all K tiles finishes the head: no barrier, no LDS
             float lo, hi;
             if (!splitk_exchange_sum_per_head(psum[0], &lo, &hi, N, ct, kt, ktiles, partials, counters)) return;
             const int head = ct * (kTileCols / kHeadDim) + (tid >> 7);
-            qk_norm_rope_head_with<true>(f32_to_bf16(lo), f32_to_bf16(hi), head, lane, rope, rope_pos, rope_gain_a,
-                                   rope_gain_b);
+            qk_norm_rope_head_at<true>(f32_to_bf16(lo), f32_to_bf16(hi), head, lane, rope, rope_pos, rope_gain_a,
+                                       rope_gain_b, rope_sin, rope_cos);
         }
     }
 }

@@ -60,10 +60,17 @@ __device__ __forceinline__ void rope_store(uint16_t* p, uint16_t v) {
 // `pos`, `gain_a` and `gain_b` are *t.pos and elements lane and lane + 64 of the head's gain (q_gain for a
 // query head, k_gain for a key head, unused for a value head): a caller that knows early which head
 // a wave will serve loads them ahead of time.
+// Sine and cosine of the rotation of elements lane and lane + 64 at position `pos`: they depend on nothing a GEMV
+// computes, so a kernel that ends with the rotation can have them ready long before.
+__device__ __forceinline__ void rope_angle(const RopeTarget& t, int pos, int lane, float* s, float* c) {
+    const float freq = exp2f(-t.log2_theta * static_cast<float>(lane) / 64.0f);
+    rope_sincos(static_cast<float>(pos) * freq, s, c);
+}
+
 template <bool WRITE_THROUGH = false>
-__device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t b_bits, int head, int lane,
-                                                       const RopeTarget& t, int pos, uint16_t gain_a,
-                                                       uint16_t gain_b) {
+__device__ __forceinline__ void qk_norm_rope_head_at(uint16_t a_bits, uint16_t b_bits, int head, int lane,
+                                                     const RopeTarget& t, int pos, uint16_t gain_a,
+                                                     uint16_t gain_b, float s, float c) {
     const bool row_ok = static_cast<unsigned>(pos) < static_cast<unsigned>(t.cache_positions);
     if (head >= t.n_q + t.n_kv) {  // value head: straight into the cache
         if (row_ok) {
@@ -83,9 +90,6 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
     // the norm output is a bf16 tensor in the usual formulation; the rotation starts from that
     const float xa = bf16_to_f32(f32_to_bf16(na));
     const float xb = bf16_to_f32(f32_to_bf16(nb));
-    const float freq = exp2f(-t.log2_theta * static_cast<float>(lane) / 64.0f);
-    float s, c;
-    rope_sincos(static_cast<float>(pos) * freq, &s, &c);
     const float oa = xa * c - xb * s;
     const float ob = xb * c + xa * s;
     // two guarded stores rather than one store through a selected pointer (see qk_norm_rope_head)
@@ -98,6 +102,16 @@ __device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t
         rope_store<WRITE_THROUGH>(dst + lane, f32_to_bf16(oa));
         rope_store<WRITE_THROUGH>(dst + lane + 64, f32_to_bf16(ob));
     }
+}
+
+// The same with the angle worked out here.
+template <bool WRITE_THROUGH = false>
+__device__ __forceinline__ void qk_norm_rope_head_with(uint16_t a_bits, uint16_t b_bits, int head, int lane,
+                                                       const RopeTarget& t, int pos, uint16_t gain_a,
+                                                       uint16_t gain_b) {
+    float s, c;
+    rope_angle(t, pos, lane, &s, &c);
+    qk_norm_rope_head_at<WRITE_THROUGH>(a_bits, b_bits, head, lane, t, pos, gain_a, gain_b, s, c);
 }
 
 // The same with the three operands loaded here.
