@@ -241,8 +241,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         const int pl = (wave * TPW + t) * 16 + mc;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const int head = 4 * mb + v;
-            if (head < G) s_score[head][pl] = (p0 + pl < ctx) ? d[v] * scale : -INFINITY;
+            // rows past G exist in s_score and nobody reads them: no test, no branch around the store
+            s_score[4 * mb + v][pl] = (p0 + pl < ctx) ? d[v] * scale : -INFINITY;
         }
     }
     __syncthreads();
@@ -335,15 +335,31 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         }
     }
     // the lane holds heads 4 mb .. 4 mb + 3 of dim `col`
+    // One test on the kind of store and one on the lane's heads around all eight stores: inside the loops they
+    // had become two branches per store.  (A lane's four heads are all live or all past G when G is a multiple
+    // of four; other groupings take the per-head test.)
+    const bool all_four = 4 * mb + 3 < G;
+    if (one_sequence && all_four) {
 #pragma unroll
-    for (int n = 0; n < 2; n++) {
-        const int col = 16 * (2 * wave + n) + mc;
+        for (int n = 0; n < 2; n++) {
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int head = 4 * mb + v;
-            if (head < G) {
-                if (one_sequence) store_result(out_base + head * kHeadDim + col, dacc[n][v]);
-                else out_base[head * kHeadDim + col] = dacc[n][v];
+            for (int v = 0; v < 4; v++) {
+                store_result(out_base + (4 * mb + v) * kHeadDim + 16 * (2 * wave + n) + mc, dacc[n][v]);
+            }
+        }
+    } else if (all_four) {
+#pragma unroll
+        for (int n = 0; n < 2; n++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) out_base[(4 * mb + v) * kHeadDim + 16 * (2 * wave + n) + mc] = dacc[n][v];
+        }
+    } else {
+#pragma unroll
+        for (int n = 0; n < 2; n++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int head = 4 * mb + v;
+                if (head < G) out_base[head * kHeadDim + 16 * (2 * wave + n) + mc] = dacc[n][v];
             }
         }
     }
