@@ -337,7 +337,9 @@ int kx_argmax_bf16(const uint16_t* x, int32_t n, int32_t* out_index, void* strea
  * The same for `batch` (1 .. KX_MAX_BATCH) sequences decoded together.  Row b of every activation
  * tensor belongs to sequence b; sequence b has its own position pos[b] and its own cache pair, which
  * starts b * cache_stride elements into k_cache / v_cache (cache_stride a multiple of 8 and at least
- * positions * n_kv_heads * 128).  Per sequence the arithmetic is that of the one-sequence calls, bit for bit.
+ * positions * n_kv_heads * 128).  Per sequence the arithmetic is that of the one-sequence calls, bit for bit;
+ * only the attention of four or more sequences splits a cache of up to 5120 positions into chunks of 128
+ * positions where the one-sequence call takes 64, and agrees with it to rounding.
  *   kx_qk_norm_rope_batch_bf16   qkv [batch, (n_q + 2 n_kv) * 128], q_out [batch, n_q * 128]
  *   kx_attn_decode_batch_bf16    q, out [batch, n_q * 128]; workspace of batch *
  *                                kx_attn_decode_workspace_bytes(...) bytes

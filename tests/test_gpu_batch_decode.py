@@ -1,8 +1,11 @@
 """Several sequences decoded together (2 <= B <= 16): the batched rotation, attention, embedding and argmax
-entry points against the one-sequence calls, bit for bit, and the batched decode step against B one-sequence
+entry points against the one-sequence calls, bit for bit (the attention from four sequences on, where it
+chunks a short cache differently, to rounding), and the batched decode step against B one-sequence
 models stepped on their own (the GEMVs of a batch run on the matrix-core kernel, those of one sequence on the
 vector kernel: equal to the rounding of fp32 sums in a different order, relative L2 <= 1e-2 on the logits of a
 two-layer model)."""
+import math
+
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -62,7 +65,14 @@ def test_batched_rotation_and_attention_equal_the_one_sequence_calls(capi, torch
         capi.attn_decode_bf16(qb, kc1[b], vc1[b], ob, n_q, n_kv, pos[b:b + 1], max_pos, ws1)
         torch.cuda.synchronize()
         assert torch.equal(bits(q[b], torch), bits(qb[0], torch)), f"q of sequence {b}"
-        assert torch.equal(bits(out[b], torch), bits(ob[0], torch)), f"attention of sequence {b}"
+        if B < 4 or max_pos > 5120:
+            assert torch.equal(bits(out[b], torch), bits(ob[0], torch)), f"attention of sequence {b}"
+        else:
+            # from four sequences on the batched call splits a short cache into chunks of 128 positions, the
+            # one-sequence call into chunks of 64: the same sums in another order
+            got, ref = out[b].float(), ob[0].float()
+            assert ((got - ref).norm() / ref.norm()).item() <= 3e-3, f"attention of sequence {b}"
+            assert (got - ref).abs().max().item() <= 2 * 2.0 ** (math.floor(math.log2(ref.abs().max().item())) - 7)
     assert torch.equal(bits(kc, torch), bits(kc1, torch))
     assert torch.equal(bits(vc, torch), bits(vc1, torch))
 
