@@ -360,7 +360,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
 #pragma unroll
             for (int m = 0; m < MB; m++) {
                 const float gt = bf16_to_f32(own_a[m]);
-                const float act = bf16_to_f32(f32_to_bf16(gt / (1.0f + expf(-gt))));
+                const float act = silu_rounded_to_bf16(gt);
                 const uint16_t xv = f32_to_bf16(act * bf16_to_f32(own_b[m]));
                 s_x[m][tid] = (stager && m0 + m < M) ? xv : static_cast<uint16_t>(0);
             }

@@ -262,7 +262,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
                 if constexpr (PRO == kProSwiGLU) {
 #pragma unroll
                     for (int j = 0; j < 8; j++) {
-                        const float act = bf16_to_f32(f32_to_bf16(av[j] / (1.0f + expf(-av[j]))));
+                        const float act = silu_rounded_to_bf16(av[j]);
                         out[j] = live ? act * bv[j] : 0.0f;
                     }
                 } else {

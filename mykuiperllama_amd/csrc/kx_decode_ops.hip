@@ -463,7 +463,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             // silu(g) is a bf16 tensor before it meets `up` in the usual formulation
-            const float act = bf16_to_f32(f32_to_bf16(g[i] / (1.0f + expf(-g[i]))));
+            const float act = silu_rounded_to_bf16(g[i]);
             g[i] = act * u[i];
         }
         reinterpret_cast<uint4*>(out)[c] = pack8(g);
