@@ -46,7 +46,7 @@ METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
 # reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).  Counters cannot be
 # read from inside this process, so the figure is carried over from that profile and named as such.
-TRAFFIC_BYTES_PER_LAUNCH = 15288300
+TRAFFIC_BYTES_PER_LAUNCH = 15337180
 TRAFFIC_SOURCE = "profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md"
 
 
