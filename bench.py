@@ -407,9 +407,7 @@ def main():
     kernel_variants = None
     if not args.no_per_shape:
         kernel_variants = {"unit": "us per launch, M = 1, cold weights, median of 10 replays of a 60-launch graph",
-                           "kernels": {"vector": "policy 1", "mfma": "policy 2 (one-shot MFMA)",
-                                       "stream": "policy 3 (resident workgroups, K loop)",
-                                       "wide": "policy 4 (16-byte cooperative loads through LDS)"}}
+                           "kernels": {"vector": "policy 1", "mfma": "policy 2 (one-shot MFMA)"}}
         for label, (K, N) in {"q_proj": (4096, 4096), "gate_proj": (4096, 12288), "gate+up fused": (4096, 24576),
                               "32B down_proj": (25600, 5120), "32B gate+up fused": (5120, 51200)}.items():
             vsets = [WeightSet(torch, {label: (K, N)}, group, gen).t[label] for _ in range(WEIGHT_SETS)]
@@ -417,9 +415,7 @@ def main():
             yv = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
             wsv = capi.make_workspace(1, K, N)
             row = {}
-            # the profiling builds have their hooks in the two product kernels only
-            variants = (("vector", 1), ("mfma", 2)) if profiling_build else (("vector", 1), ("mfma", 2), ("stream", 3), ("wide", 4))
-            for name, policy in variants:
+            for name, policy in (("vector", 1), ("mfma", 2)):
                 capi.set_awq_kernel_policy(policy)
 
                 def launch_v(first, count, vsets=vsets, xv=xv, yv=yv, wsv=wsv):

@@ -44,7 +44,10 @@ extern "C" {
 
 #define KX_MAX_BATCH 16            /* largest M the GEMV entry points take */
 
-/* ABI version; bumped when a signature changes. */
+/* ABI version; bumped when a signature or the layout of a struct below changes.  kx_abi_version() is what the
+ * loaded library was built as: a binding compares it with the KX_ABI_VERSION it was compiled against before it
+ * calls anything else (kx_chain_desc has no size field; a library of another version reads other fields). */
+#define KX_ABI_VERSION 3
 int kx_abi_version(void);
 
 /* Static, human-readable text for a return code of this library (KX_ERR_* or hipError_t). */
@@ -85,12 +88,14 @@ int kx_gemv_awq_bf16(const uint16_t* x, const int32_t* qweight, const uint16_t* 
 
 /* kx_gemv_awq_bf16 for callers that cannot allocate or hand over a workspace (code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc): the split-K workspace is a static device array inside
- * the library, kx_gemv_awq_static_scratch_bytes() bytes (256 KiB of counters + 8 MiB of partial sums) per GPU
+ * the library, kx_gemv_awq_static_scratch_bytes() bytes (512 KiB of counters and slots + 8 MiB of partial sums) per GPU
  * the library runs on, held until the process ends.  Same arguments, kernels and bits as kx_gemv_awq_bf16.
  * A shape whose kx_gemv_workspace_bytes(M, K, N) exceeds the array is rejected with KX_ERR_WORKSPACE and
- * nothing is launched (every Qwen3-8B and -32B projection fits at M = 1, the 8B ones up to M = 4).
+ * nothing is launched (every Qwen3-8B and -32B projection fits at M = 1, the seven separate 8B ones up to
+ * M = 4; the fused 8B gate|up 4096 -> 24576 fits up to M = 2, the 32B-shaped fused gate|up 5120 -> 51200 at M = 1 only).
  * Calls no hipMalloc / hipFree.  The first call on a device looks the array's address up and enqueues
- * one small kernel that zeroes the counters; make that call outside stream capture.  All calls on one GPU
+ * one small kernel that zeroes the counters (the array is zero when the library is loaded, so that kernel
+ * restates what already holds); make that call outside stream capture all the same.  All calls on one GPU
  * share that GPU's array: calls that may overlap (different streams) race - use kx_gemv_awq_bf16 with
  * separate workspaces for those.
  * Reference counterpart: none (the reference has no split reduction and allocates through

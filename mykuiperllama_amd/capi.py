@@ -14,6 +14,8 @@ _I32 = ctypes.c_int32
 _I64 = ctypes.c_int64
 _SZ = ctypes.c_size_t
 
+ABI_VERSION = 3  # KX_ABI_VERSION of the include/kx_hip.h this file mirrors
+
 # name -> (restype, argtypes); mirrors include/kx_hip.h declaration by declaration
 SIGNATURES = {
     "kx_abi_version": (ctypes.c_int, []),
@@ -110,6 +112,10 @@ def load(path=None):
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
+    built_as = lib.kx_abi_version()
+    if built_as != ABI_VERSION:
+        raise RuntimeError(f"{lib_path} was built as ABI version {built_as}, this binding mirrors version "
+                           f"{ABI_VERSION} of include/kx_hip.h (ChainDesc would not match kx_chain_desc)")
     _lib = lib
     return lib
 
@@ -172,7 +178,9 @@ def workspace_bytes(M, K, N):
 def make_workspace(M, K, N, device="cuda"):
     """Allocate and initialise a workspace large enough for a GEMV of this shape."""
     import torch
-    nbytes = max(workspace_bytes(M, K, N), 262144)
+    nbytes = workspace_bytes(M, K, N)  # the zeroed area of every workspace plus the shape's partial sums
+    if nbytes == 0:
+        raise ValueError(f"no GEMV takes M={M}, K={K}, N={N}")
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
     _check(load().kx_workspace_init(ws.data_ptr(), nbytes, _stream()))
     return ws
@@ -242,11 +250,11 @@ _policy = 0
 def set_awq_kernel_policy(policy):
     """Test and benchmark plumbing: which kernel gemv_awq_bf16 of THIS module asks for from now on.
     0 = the product entry point (the library chooses by shape); 1 = vector-ALU kernel, 2 = one-shot MFMA
-    kernel, 3 / 4 = the two measured alternatives (K-loop kernel, wide-load kernel), each through the internal entry point kx_gemv_awq_bf16_policy.
+    kernel, each through the internal entry point kx_gemv_awq_bf16_policy.
     The library itself keeps no such state."""
     global _policy
-    if policy not in (0, 1, 2, 3, 4):
-        raise ValueError("policy must be 0 .. 4")
+    if policy not in (0, 1, 2):
+        raise ValueError("policy must be 0, 1 or 2")
     _policy = policy
 
 

@@ -1,8 +1,6 @@
 // Host side of the fused INT4 AWQ dequantise + GEMV: shape checks, launch plan, C ABI.
 #include "kx_awq_gemv_kernel.h"
 #include "kx_awq_gemv_mfma_kernel.h"
-#include "kx_awq_gemv_stream_kernel.h"
-#include "kx_awq_gemv_wide_kernel.h"
 #include "kx_internal.h"
 
 #include <mutex>
@@ -106,90 +104,54 @@ inline AwqPlan make_valu_plan(int M, int K, int N, bool allow_long_rows = true, 
     return p;
 }
 
+// One activation row, plain store, the K tiles meeting in fixed point (splitk_exchange_store_fixed): that
+// exchange costs about half of the one above per K tile, which moves the choice towards smaller workgroups -
+// four waves of sixteen rows (128 rows of K, 256 threads) join the candidates.  Measured, us per launch with
+// 128 / 256 / 512 / 384 rows per workgroup: k 4096->1024 3.65 / 3.85 / 4.72 / -, q 4096->4096 4.47 / 4.55 /
+// 5.10 / -, q|k|v 4096->6144 5.19 / 5.52 / 5.38 / -, gate 4096->12288 8.16 / 7.63 / 8.34 / -, gate|up
+// 4096->24576 13.67 / 12.81 / 12.82 / -, down 12288->4096 - / 7.75 / 8.61 / 7.28, 32B-shaped o 8192->5120
+// - / 7.10 / 8.03 / -.  ktiles == 1 in the result means that the exchange does not apply (a single K tile, more
+// K tiles than the slot's arrival count holds, or more columns than the zeroed area has slots for).
+constexpr int kFixedExchangeRows = 4;
+
+inline AwqPlan make_fixed_plan(int K, int N) {
+    AwqPlan p{};
+    p.mfma = false;
+    p.coltiles = (N / 8 + kWC - 1) / kWC;
+    p.mb = 1;
+    p.mtiles = 1;
+    p.waves = 8;
+    p.rt = 16;
+    p.ktiles = 1;
+    if (static_cast<size_t>(N) * 16 > kCounterBytes) return p;  // a slot and a mask word per column
+    const struct { int waves, rt; } shapes[4] = {{8, 16}, {4, 16}, {8, 32}, {12, 16}};
+    long best = -1;
+    for (const auto& c : shapes) {
+        const int rows = rows_per_block(c.waves, c.rt);
+        if (K < rows || ((c.waves != 8 || c.rt != 16) && K % rows != 0)) continue;
+        const long kt = (K + rows - 1) / rows;
+        if (kt < 2 || kt > kFixedMaxKTiles) continue;
+        const long blocks = static_cast<long>(p.coltiles) * kt;
+        const long cost = (blocks + kComputeUnits - 1) / kComputeUnits * rows + kFixedExchangeRows * kt;
+        if (best < 0 || cost < best) {
+            best = cost;
+            p.waves = c.waves;
+            p.rt = c.rt;
+            p.ktiles = static_cast<int>(kt);
+        }
+    }
+    return p;
+}
+
 inline AwqPlan make_plan(int M, int K, int N, int group, int mode) {
     // The MFMA kernel needs quantisation groups that tile the workgroup's K range (powers of two)
     // and loads two packed words at a time (N a multiple of sixteen).
     const bool mfma_ok = is_pow2(group) && (N % 16) == 0;  // mfma_shape_ok() below
-    // One activation row stays on the vector kernel although the MFMA kernel is a few per cent faster on
-    // wide projections (us per launch, vector / MFMA: 4096->12288 8.9 / 8.5, 4096->24576 13.5 / 13.0,
-    // 5120->51200 30.9 / 29.3; narrow and tall ones the other way round: 4096->4096 5.7 / 5.8, 12288->4096
-    // 9.2 / 9.6): the launches with an activation prologue run on the vector kernel, and a plain launch
-    // returns their bits only if it adds in the same order.
+    // One activation row stays on the vector kernel: with the fixed-point exchange it is ahead of the MFMA kernel on
+    // every measured shape (kx_gemv_awq_bf16_policy decides that before it comes here), and the launches with an
+    // activation prologue or an epilogue live in it.
     const bool mfma = mfma_ok && (mode == KX_POLICY_MFMA || (mode == KX_POLICY_BY_SHAPE && M >= 2));
     return mfma ? make_mfma_plan(M, K, N, group) : make_valu_plan(M, K, N);
-}
-
-// The wide-load MFMA kernel: power-of-two groups of at least 32 rows, N a multiple of 32 (a thread loads
-// four packed words at a time), four waves of one or two 32-row steps per workgroup.
-inline bool wide_ok(int K, int N, int group) {
-    return is_pow2(group) && group >= kStepRows && (N % 32) == 0 && (K % 8) == 0;
-}
-
-inline AwqPlan make_wide_plan(int M, int K, int N, int group) {
-    AwqPlan p;
-    p.mfma = true;
-    p.coltiles = (N + kTileCols - 1) / kTileCols;
-    p.mb = M;
-    p.mtiles = 1;
-    p.waves = kWideWaves;
-    int ks = 2;
-    while (ks > 1 && (ks * kStepRows > group || p.waves * ks * kStepRows > K)) ks /= 2;
-    p.rt = ks;
-    const int kb = p.waves * ks * kStepRows;
-    p.ktiles = (K + kb - 1) / kb;
-    return p;
-}
-
-// The streaming kernel: up to four activation rows, power-of-two groups, whole column tiles, and a run
-// per workgroup that holds at least one 32-row step per wave and at most one tile boundary.
-struct StreamPlan {
-    bool ok;
-    int waves;     // waves per workgroup
-    int grid;      // workgroups, at most one per compute unit
-    int steps;     // 32-row steps per column tile
-    int units;     // column tiles * steps
-    int slots;     // most workgroups that share one column tile
-};
-
-inline StreamPlan make_stream_plan(int M, int K, int N, int group) {
-    StreamPlan p{};
-    p.waves = 8;
-    const size_t weight_bytes = static_cast<size_t>(K) * N / 2;
-    p.ok = M >= 1 && M <= 4 && is_pow2(group) && group >= kStepRows && (N % kTileCols) == 0 && (K % kStepRows) == 0 &&
-           K >= 8 * kStepRows && N / kTileCols <= kMaxStreamGrid &&
-           weight_bytes < (static_cast<size_t>(1) << 31) && static_cast<size_t>(M) * K * 2 < (static_cast<size_t>(1) << 31) &&
-           static_cast<size_t>(N / kTileCols) * (K / kStepRows) < (static_cast<size_t>(1) << 24);
-    if (!p.ok) return p;
-    const int coltiles = N / kTileCols;
-    p.steps = K / kStepRows;
-    p.units = coltiles * p.steps;
-    int grid = p.units / 8;
-    if (grid > kMaxStreamGrid) grid = kMaxStreamGrid;
-    if (grid < coltiles) grid = coltiles;
-    p.grid = grid;
-    p.slots = p.steps / (p.units / grid) + 2;
-    return p;
-}
-
-// n / d == (n * m) >> sh for every 0 <= n < 2^24: m = ceil(2^(24 + L) / d) with 2^L >= d
-inline void stream_magic(int d, uint32_t* m, int* sh) {
-    int L = 0;
-    while ((1 << L) < d) L++;
-    *sh = 24 + L;
-    const unsigned long long one = static_cast<unsigned long long>(1) << *sh;
-    *m = static_cast<uint32_t>((one + static_cast<unsigned long long>(d) - 1) / static_cast<unsigned long long>(d));
-}
-
-template <int VR>
-void launch_stream_vr(const StreamPlan& p, const StreamArgs& a, hipStream_t stream) {
-    // eight waves, one unit in flight beside the one being worked on: the best of the depths and wave counts measured
-    hipLaunchKernelGGL((awq_gemv_stream_kernel<8, VR, 2>), dim3(p.grid), dim3(8 * kWave), stream_lds_bytes(8, VR), stream, a);
-}
-
-inline void launch_stream(const StreamPlan& p, const StreamArgs& a, hipStream_t stream) {
-    if (a.M == 1) launch_stream_vr<1>(p, a, stream);
-    else if (a.M == 2) launch_stream_vr<2>(p, a, stream);
-    else launch_stream_vr<4>(p, a, stream);
 }
 
 template <int WAVES, int RT>
@@ -342,11 +304,10 @@ extern "C" size_t kx_gemv_workspace_bytes(int32_t M, int32_t K, int32_t N) {
     const int kt_valu = kx::make_valu_plan(M, K, N, true, false).ktiles;  // the entry points that keep 8 waves exchange more
     const int kt_mfma = kx::make_mfma_plan(M, K, N, 32).ktiles;  // the smallest group gives the most K tiles
     size_t ktiles = static_cast<size_t>(kt_valu > kt_mfma ? kt_valu : kt_mfma);
-    // the two measured alternatives (internal entry point only) size their exchange differently
-    const size_t kt_wide = static_cast<size_t>(kx::make_wide_plan(M, K, N, 32).ktiles);
-    if (kt_wide > ktiles) ktiles = kt_wide;
-    const kx::StreamPlan sp = kx::make_stream_plan(M, K, N, 32);  // group size does not enter its slot count
-    if (sp.ok && static_cast<size_t>(sp.slots) > ktiles) ktiles = static_cast<size_t>(sp.slots);
+    if (M == 1) {
+        const size_t kt_fixed = static_cast<size_t>(kx::make_fixed_plan(K, N).ktiles);  // its slow path parks partial sums there
+        if (kt_fixed > ktiles) ktiles = kt_fixed;
+    }
     return kx::kCounterBytes + ktiles * M * static_cast<size_t>(N) * sizeof(float);
 }
 
@@ -417,6 +378,7 @@ extern "C" int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight
     if (!x) return KX_ERR_NULL_POINTER;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
     if (rc != KX_OK) return rc;
+    if (reinterpret_cast<uintptr_t>(x) % 16) return KX_ERR_ALIGNMENT;
     if (kx_gemv_workspace_bytes(M, K, N) > kStaticScratchBytes) return KX_ERR_WORKSPACE;  // larger than the static array
     void* ws = nullptr;
     rc = static_scratch_for_current_device(&ws, kx::as_stream(stream));
@@ -437,78 +399,32 @@ extern "C" int kx_gemv_awq_bf16_policy(const uint16_t* x, const int32_t* qweight
                                        const int32_t* qzeros, uint16_t* y, int32_t M, int32_t K, int32_t N,
                                        int32_t group_size, void* workspace, size_t workspace_bytes,
                                        void* stream, int32_t policy) {
-    if (policy < KX_POLICY_BY_SHAPE || policy > KX_POLICY_WIDE) return KX_ERR_BAD_SHAPE;
+    if (policy < KX_POLICY_BY_SHAPE || policy > KX_POLICY_MFMA) return KX_ERR_BAD_SHAPE;
     if (!x) return KX_ERR_NULL_POINTER;
     int rc = kx::check_awq_weights(qweight, scales, qzeros, y, M, K, N, group_size);
     if (rc != KX_OK) return rc;
     if (reinterpret_cast<uintptr_t>(x) % 16) return KX_ERR_ALIGNMENT;
-    if (policy == KX_POLICY_STREAM && kx::make_stream_plan(M, K, N, group_size).ok) {
-        const kx::StreamPlan sp = kx::make_stream_plan(M, K, N, group_size);
-        if (reinterpret_cast<uintptr_t>(qweight) % 8 || reinterpret_cast<uintptr_t>(qzeros) % 8) return KX_ERR_ALIGNMENT;
-        const bool tiles_shared = sp.grid != N / kx::kTileCols;  // else every workgroup owns one whole tile
-        if (tiles_shared) {
-            if (!workspace) return KX_ERR_WORKSPACE;
-            if (reinterpret_cast<uintptr_t>(workspace) % 256) return KX_ERR_ALIGNMENT;
-            const size_t need = kx::kCounterBytes + static_cast<size_t>(sp.slots) * M * N * sizeof(float);
-            if (workspace_bytes < need) return KX_ERR_WORKSPACE;
-        }
-        int group_shift = 0;
-        while ((1 << group_shift) < group_size) group_shift++;
-        kx::StreamArgs a{};
-        a.x = x;
-        a.qweight = reinterpret_cast<const uint32_t*>(qweight);
-        a.scales = scales;
-        a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
-        a.y = y;
-        a.counters = tiles_shared ? static_cast<uint32_t*>(workspace) : nullptr;
-        a.partials = tiles_shared ? reinterpret_cast<float*>(static_cast<char*>(workspace) + kx::kCounterBytes) : nullptr;
-        a.M = M;
-        a.K = K;
-        a.N = N;
-        a.group_shift = group_shift;
-        a.S = sp.steps;
-        a.U = sp.units;
-        a.G = sp.grid;
-        a.lo = sp.units / sp.grid;
-        a.rem = sp.units % sp.grid;
-        kx::stream_magic(a.S, &a.mS, &a.shS);
-        kx::stream_magic(a.lo, &a.mlo, &a.shlo);
-        kx::stream_magic(a.lo + 1, &a.mlo1, &a.shlo1);
-        kx::launch_stream(sp, a, kx::as_stream(stream));
-        return kx::launch_status();
-    }
-    if (policy == KX_POLICY_WIDE && kx::wide_ok(K, N, group_size)) {
-        if (reinterpret_cast<uintptr_t>(qweight) % 16 || reinterpret_cast<uintptr_t>(qzeros) % 16) return KX_ERR_ALIGNMENT;
-        const kx::AwqPlan p = kx::make_wide_plan(M, K, N, group_size);
-        float* partials = nullptr;
-        uint32_t* counters = nullptr;
-        rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
-        if (rc != KX_OK) return rc;
-        int group_shift = 0;
-        while ((1 << group_shift) < group_size) group_shift++;
-        hipStream_t s = kx::as_stream(stream);
-#define KX_WARGS x, qweight, scales, qzeros, y, partials, counters, M, K, N, group_shift, p.coltiles, p.ktiles, s
-#define KX_WIDE_BY_M(KS)                                                        \
-    do {                                                                        \
-        if (M == 1) kx::launch_awq_gemv_wide<KS, 1, 1>(KX_WARGS);               \
-        else if (M == 2) kx::launch_awq_gemv_wide<KS, 2, 1>(KX_WARGS);          \
-        else if (M <= 4) kx::launch_awq_gemv_wide<KS, 4, 1>(KX_WARGS);          \
-        else if (M <= 8) kx::launch_awq_gemv_wide<KS, 8, 1>(KX_WARGS);          \
-        else kx::launch_awq_gemv_wide<KS, 8, 2>(KX_WARGS);                      \
-    } while (0)
-        if (p.rt == 2) KX_WIDE_BY_M(2);
-        else KX_WIDE_BY_M(1);
-#undef KX_WIDE_BY_M
-#undef KX_WARGS
-        return kx::launch_status();
-    }
-    kx::AwqPlan p = kx::make_plan(M, K, N, group_size,
-                                  policy == KX_POLICY_STREAM || policy == KX_POLICY_WIDE ? KX_POLICY_BY_SHAPE : policy);
     float* partials = nullptr;
     uint32_t* counters = nullptr;
+    hipStream_t s = kx::as_stream(stream);
+    if (M == 1 && policy == KX_POLICY_BY_SHAPE) {
+        // one activation row, plain store: the K tiles of a column meet in a 64-bit fixed-point word
+        const kx::AwqPlan fp = kx::make_fixed_plan(K, N);
+        if (fp.ktiles > 1) {
+            rc = kx::resolve_workspace(fp, 1, N, workspace, workspace_bytes, &partials, &counters);
+            if (rc != KX_OK) return rc;
+#define KX_FARGS x, qweight, scales, qzeros, y, partials, counters, 1, K, N, group_size, fp.coltiles, fp.ktiles, 1, s
+            if (fp.rt == 32) kx::launch_awq_gemv<8, 32, 1, kx::kProNone, kx::kEpiStoreFixed>(KX_FARGS);
+            else if (fp.waves == 12) kx::launch_awq_gemv<12, 16, 1, kx::kProNone, kx::kEpiStoreFixed>(KX_FARGS);
+            else if (fp.waves == 8) kx::launch_awq_gemv<8, 16, 1, kx::kProNone, kx::kEpiStoreFixed>(KX_FARGS);
+            else kx::launch_awq_gemv<4, 16, 1, kx::kProNone, kx::kEpiStoreFixed>(KX_FARGS);
+#undef KX_FARGS
+            return kx::launch_status();
+        }
+    }
+    kx::AwqPlan p = kx::make_plan(M, K, N, group_size, policy);
     rc = kx::resolve_workspace(p, M, N, workspace, workspace_bytes, &partials, &counters);
     if (rc != KX_OK) return rc;
-    hipStream_t s = kx::as_stream(stream);
     if (p.mfma) {
         int group_shift = 0;
         while ((1 << group_shift) < group_size) group_shift++;

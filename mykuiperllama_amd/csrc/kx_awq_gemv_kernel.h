@@ -91,7 +91,8 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     uint16_t* __restrict__ y, float* __restrict__ partials, uint32_t* __restrict__ counters,
-    int M, int K, int N, int group, int coltiles, int ktiles, FusedInput fi, RopeTarget rope, ResidualTarget res) {
+    int M, int K, int N, int group, int group_shift, int coltiles, int ktiles, FusedInput fi, RopeTarget rope,
+    ResidualTarget res) {
     constexpr int SLOTS = WAVES * kSlotsPerWave;
     constexpr int KB = SLOTS * RT;
     constexpr int THREADS = WAVES * kWave;
@@ -115,10 +116,15 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     __shared__ float s_norm[MERGE ? HB : 1];
     __shared__ float s_mpart[MERGE ? kMergeParts : 1][MERGE ? KB : 1];
 
+    // The pointers of the epilogue are fetched with the other kernel arguments: left to itself the compiler loads
+    // them where they are first used, a scalar-memory round trip behind the reduction.
+    asm volatile("" ::"s"(y), "s"(partials), "s"(counters));
     const int tid = threadIdx.x;
-    const int ct = blockIdx.x % coltiles;
-    const int kt = blockIdx.x / coltiles;
-    const int m0 = blockIdx.y * MB;
+    // grid = (column tiles, K tiles, activation-row tiles): x runs fastest, so workgroups that start together read
+    // neighbouring 128-byte pieces of the same rows, and no division stands in front of the first load
+    const int ct = blockIdx.x;
+    const int kt = blockIdx.y;
+    const int m0 = blockIdx.z * MB;
     const int nw = N >> 3;
 
     const int wc = tid % kWC;       // word column inside the tile
@@ -228,6 +234,25 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         }
     }
 
+    // Fixed-point exchange: what the unit of a column is made of (kx_splitk_exchange.h) is requested ahead of the
+    // weights and summed while they are on their way.  Every wave that will own columns (threads 0..255) reads the
+    // same sample of the activation row - eight spread-out runs of 128 bytes, 512 elements - and the scale of its
+    // column in group 0; the wave sum needs no LDS and is the same bits in every workgroup of the launch.
+    constexpr bool FIXED = EPI == kEpiStoreFixed;
+    static_assert(!FIXED || (MB == 1 && PRO == kProNone), "the fixed-point exchange serves the plain one-row launch");
+    FixedUnit fixed_unit{1.0f, 1.0f};
+    u32x4 fixed_xs = {0u, 0u, 0u, 0u};
+    uint16_t fixed_sref = 0;
+    if constexpr (FIXED) {
+        // every wave loads, also those that will own no column: a branch here would make every later wait a wait
+        // for all loads
+        const int pieces = K >> 3;                         // 16-byte pieces of the row, at least four (K >= 32)
+        const int run = (tid % kWave) >> 3;                // eight runs of eight pieces
+        const int pc = static_cast<int>((static_cast<long>(run) * pieces) >> 3) + (tid & 7);
+        fixed_xs = *reinterpret_cast<const u32x4*>(x + 8 * (pc < pieces ? pc : pieces - 1));
+        const int col = ct * kTileCols + tid % kTileCols;
+        fixed_sref = scales[col < N ? col : N - 1];
+    }
     // Small, cache-resident operands first, then every weight load of this lane, all of them
     // issued before anything is consumed: loads return in order, so the arithmetic on row r
     // can start while rows r+1.. are still in flight.
@@ -238,10 +263,12 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     uint4 sraw = make_uint4(0u, 0u, 0u, 0u);
     uint4 xraw[MB][RT / 8];
     uint32_t w[RT];
-    if (STAGED || active) {
-        const int ld_wcg = STAGED ? (wcg < nw ? wcg : nw - 1) : wcg;
-        const int ld_k0 = STAGED ? (k0 < K ? k0 : K - RT) : k0;
-        const int g = ld_k0 / group;
+    constexpr bool CLAMPED = STAGED || FIXED;  // loads at clamped addresses instead of a branch around them
+    if (CLAMPED || active) {
+        const int ld_wcg = CLAMPED ? (wcg < nw ? wcg : nw - 1) : wcg;
+        const int ld_k0 = CLAMPED ? (k0 < K ? k0 : K - RT) : k0;
+        // power-of-two groups (the usual case) by a shift: a division is some forty instructions ahead of the loads
+        const int g = group_shift >= 0 ? ld_k0 >> group_shift : ld_k0 / group;
         // On the plain launch scales and zero points carry the weights' streaming hint: measured + 1 % on the
         // seven-projection step; on the launches of the decode step the same hint cost 0.4 %.
         if constexpr (PRO == kProNone) {
@@ -259,7 +286,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
                 for (int r8 = 0; r8 < RT / 8; r8++) {
                     // rows past M read row M - 1 and are zeroed: no branch between the loads
                     const int mrow = m0 + m < M ? m0 + m : M - 1;
-                    const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(mrow) * K + k0 + 8 * r8);
+                    const uint4 got = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(mrow) * K + ld_k0 + 8 * r8);
                     xraw[m][r8] = (m == 0 || m0 + m < M) ? got : make_uint4(0u, 0u, 0u, 0u);
                 }
             }
@@ -289,6 +316,18 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
             }
         }
         // keep the scheduler from sinking loads below the first use of an earlier one
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (FIXED) {
+        const uint32_t pw[4] = {fixed_xs.x, fixed_xs.y, fixed_xs.z, fixed_xs.w};
+        float xa = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) xa = dot2_bf16(pw[i] & 0x7fff7fffu, 0x3F803F80u, xa);
+        // the sample stands for the whole row: K / 512 elements per element read
+        fixed_unit = fixed_unit_of(wave_sum(xa) * (static_cast<float>(K) * (1.0f / 512.0f)) *
+                                   __builtin_fabsf(f16_bits_to_f32(fixed_sref)));
+        // pinned here: left to itself the compiler sinks this arithmetic to its one use, behind the reduction
+        asm volatile("" : "+v"(fixed_unit.unit), "+v"(fixed_unit.inv_unit));
         __builtin_amdgcn_sched_barrier(0);
     }
     // The rotation's sine and cosine while the weights are on their way: the vector unit has nothing to do yet,
@@ -424,7 +463,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         lds_barrier();
     }
 
-    if (active) {
+    if (FIXED || active) {
         // Two rows at a time: the codes of rows k and k+1 of one column become a pair of bf16 numbers
         // 16 + q (exponent of 16.0, the code in the top four mantissa bits), the activations of the two
         // rows already lie in memory as such a pair, and one dot-product instruction does both
@@ -439,6 +478,9 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         // converted here does not stand between the last weight row and the reduction.  With 32 rows per lane the
         // sixteen registers this keeps across the loop cost more than the shorter tail gains (measured), and
         // the conversion stays behind the loop.
+        // The fixed-point launch has no branch around its loads or its arithmetic: lanes outside the matrix work on
+        // what their clamped addresses hold and contribute through a scale of zero.
+        auto lane_scale = [&](float sc) { return (FIXED && !active) ? 0.0f : sc; };
         constexpr bool kConvertEarly = RT <= 16;
         float col_scale[8], col_zoff[8];
         if constexpr (kConvertEarly) {
@@ -448,7 +490,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
 #pragma unroll
             for (int c = 0; c < 8; c++) {
                 const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
-                col_scale[c] = f16_bits_to_f32(bits);
+                col_scale[c] = lane_scale(f16_bits_to_f32(bits));
                 col_zoff[c] = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -492,7 +534,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
 #pragma unroll
             for (int c = 0; c < 8; c++) {
                 const uint16_t bits = static_cast<uint16_t>((c & 1) ? (sw[c >> 1] >> 16) : (sw[c >> 1] & 0xffffu));
-                col_scale[c] = f16_bits_to_f32(bits);
+                col_scale[c] = lane_scale(f16_bits_to_f32(bits));
                 col_zoff[c] = __builtin_fmaf(z[c], kCodeScale, kCodeOffset);  // 16 + z, exact
             }
         }
@@ -556,11 +598,20 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
         return;
     }
 #endif
-    if constexpr (EPI == kEpiStore && MB == 1) {
+    if constexpr (EPI == kEpiStoreFixed) {
+        if (tid >= kTileCols) return;
+        if (ktiles == 1) {
+            const int col = ct * kTileCols + tid;
+            if (col < N) store_result(y + col, f32_to_bf16(psum[0]));
+            return;
+        }
+        splitk_exchange_store_fixed(psum[0], fixed_unit, N, ct, kt, ktiles,
+                                    reinterpret_cast<unsigned long long*>(counters), partials, y);
+    } else if constexpr (EPI == kEpiStore && MB == 1) {
         // one activation row (MB == 1 is M == 1 in every plan): every wave reports for itself
         splitk_exchange_store_per_wave(psum[0], N, ct, kt, ktiles, ct, partials, counters, y);
     } else if constexpr (EPI == kEpiStore) {
-        splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.y * coltiles + ct, partials, counters, y,
+        splitk_exchange_store<MB>(psum, m0, M, N, ct, kt, ktiles, blockIdx.z * coltiles + ct, partials, counters, y,
                                   &s_prev);
     } else if constexpr (EPI == kEpiResidual) {
         static_assert(MB == 1, "the residual epilogue serves one activation row");
@@ -611,12 +662,16 @@ inline void launch_awq_gemv(const uint16_t* x, const int32_t* qweight, const uin
                             int M, int K, int N, int group, int coltiles, int ktiles, int mtiles,
                             hipStream_t stream, const FusedInput& fi = FusedInput{},
                             const RopeTarget& rope = RopeTarget{}, const ResidualTarget& res = ResidualTarget{}) {
-    dim3 grid(coltiles * ktiles, mtiles, 1);
+    dim3 grid(coltiles, ktiles, mtiles);
     dim3 block(WAVES * kWave, 1, 1);
+    int group_shift = -1;  // log2(group) where it is a power of two
+    for (int sh = 0; sh < 31; sh++) {
+        if ((1 << sh) == group) group_shift = sh;
+    }
     hipLaunchKernelGGL((awq_gemv_kernel<WAVES, RT, MB, PRO, EPI>), grid, block, 0, stream, x,
                        reinterpret_cast<const uint32_t*>(qweight), scales,
                        reinterpret_cast<const uint32_t*>(qzeros), y, partials, counters, M, K, N,
-                       group, coltiles, ktiles, fi, rope, res);
+                       group, group_shift, coltiles, ktiles, fi, rope, res);
 }
 
 }  // namespace kx

@@ -14,12 +14,14 @@ constexpr int kWave = 64;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-// Workspace layout: [kCounterBytes of arrival counters, one per 64-byte line][fp32 partial sums].
-// Counters that share a line serialise at the memory side (~10 ns per atomic, measured), so
-// every (column tile, activation tile) pair gets lines of its own: four of them, one per quarter of
-// the tile, for the exchange in which every wave of 64 columns reports for itself.
+// Workspace layout: [kCounterBytes, zeroed once and left zeroed by every launch][fp32 partial sums].
+// The zeroed area holds, depending on the launch, arrival counters on 64-byte lines of their own (counters that
+// share a line serialise at the memory side, ~10 ns per atomic, measured; every (column tile, activation tile)
+// pair gets four lines, one per quarter of the tile, for the exchange in which every wave of 64 columns reports
+// for itself) or, for the fixed-point exchange of the one-row plain launch, a 64-bit slot and a 64-bit mask word
+// per output column (up to 32 768 columns).
 constexpr int kCountersPerTile = 4;
-constexpr size_t kCounterBytes = 262144;
+constexpr size_t kCounterBytes = 524288;
 constexpr int kMaxTiles = kCounterBytes / 64 / kCountersPerTile;
 
 // nibble i of a packed word holds column 8j + kOrder[i]

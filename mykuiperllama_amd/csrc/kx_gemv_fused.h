@@ -55,6 +55,7 @@ struct ResidualTarget {
 constexpr int kEpiStore = 0;   // y[m, n] = bf16(sum)
 constexpr int kEpiQkRope = 1;  // the row is q | k | v heads of 128: per-head norm, rotation, cache append (M = 1)
 constexpr int kEpiResidual = 2;  // residual add + per-tile sums of squares, see ResidualTarget
+constexpr int kEpiStoreFixed = 3;  // y[n] = bf16(sum), M = 1, the K tiles meeting in 64-bit fixed point (kx_splitk_exchange.h)
 
 }  // namespace kx
 

@@ -13,13 +13,11 @@
 extern "C" {
 #endif
 
-#define KX_POLICY_BY_SHAPE 0   /* what kx_gemv_awq_bf16 does */
-#define KX_POLICY_VECTOR 1     /* the vector-ALU kernel (any accepted shape) */
+#define KX_POLICY_BY_SHAPE 0   /* what kx_gemv_awq_bf16 does: one row on the vector kernel with the fixed-point exchange
+                                  wherever that applies, several rows on the MFMA kernel */
+#define KX_POLICY_VECTOR 1     /* the vector-ALU kernel with the ordered fp32 exchange (any accepted shape): the sums of
+                                  the launches with a prologue or an epilogue, bit for bit */
 #define KX_POLICY_MFMA 2       /* the one-shot MFMA kernel where group size and N allow, else the vector kernel */
-/* Two measured alternatives that lost against the kernels above and are kept so that the comparison can be
- * repeated (bench.py prints it): */
-#define KX_POLICY_STREAM 3     /* resident workgroups walking a K loop ("stream-K"), where it applies, else as by shape */
-#define KX_POLICY_WIDE 4       /* 16-byte cooperative loads through LDS, where it applies, else as by shape */
 
 /* kx_gemv_awq_bf16 with the kernel chosen by the caller. */
 int kx_gemv_awq_bf16_policy(const uint16_t* x, const int32_t* qweight, const uint16_t* scales,

@@ -2,7 +2,7 @@
 #include "kx_common.h"
 
 extern "C" int kx_abi_version(void) {
-    return 3;
+    return KX_ABI_VERSION;
 }
 
 extern "C" const char* kx_error_string(int code) {

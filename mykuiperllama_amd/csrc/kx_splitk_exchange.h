@@ -41,6 +41,13 @@ namespace kx {
 constexpr int kTileCols = 256;     // output columns per column tile, one thread each in the exchange
 constexpr int kCounterStride = 16; // uint32 slots between counters: one 64-byte line each
 
+// Nothing in the language orders the relaxed loads of a read-back behind the relaxed atomic whose result decides
+// that they run; the hardware does (the loads sit behind a branch on that result).  This keeps the compiler from
+// moving memory operations across the point as well: no instruction, no cache traffic.
+__device__ __forceinline__ void compiler_fence() {
+    asm volatile("" ::: "memory");
+}
+
 __device__ __forceinline__ void store_agent(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -99,6 +106,7 @@ __device__ __forceinline__ bool splitk_exchange_sum(const float (&psum)[ROWS], f
     }
     __syncthreads();
     if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return false;
+    compiler_fence();  // the read-back below stays behind the counter's return
 
     // Last to arrive: every other workgroup's partials were acknowledged before its increment.
     // The read-back is a round trip to memory (~1 us, the longest leg of the exchange), so as many
@@ -210,6 +218,7 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_wave(float psum, float* 
     uint32_t prev = 0;
     if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
+    compiler_fence();  // the read-back below stays behind the counter's return
     if (prev != static_cast<uint32_t>(ktiles - 1)) return false;
 
     // last of its quarter: every other wave's partial sums were acknowledged before its increment
@@ -279,6 +288,91 @@ __device__ __forceinline__ void splitk_exchange_store_per_wave(float psum, int N
     if (col < N) store_result(y + col, f32_to_bf16(sum));
 }
 
+// ---- One activation row, plain store: the K tiles of a column meet in one 64-bit word ----
+//
+// Every workgroup turns its partial sum of a column into a 52-bit fixed-point number and adds it to the column's
+// slot with one returning device-scope atomic; the slot's top bits count the arrivals, and the thread whose
+// atomic returns ktiles - 1 holds, in the returned word plus its own addend, the finished sum: it converts,
+// stores y and clears the slot.  One trip to memory where the exchanges above take three (store
+// acknowledgement, counter, read-back), and nothing to order: the sum travels in the atomic itself.  Integer
+// addition commutes, so the result does not depend on the order of arrival (bitwise reproducible).
+//
+// slot = [ arrivals : 6 ][ arrivals that took the slow path : 6 ][ sum of (v + 2^45) : 52 ],  |v| < 2^45
+//
+// The unit of v must be the same in every workgroup of a column and is therefore a function of operands that
+// all of them can read: unit = 2^ceil(log2(16 * 256 * sum_k |x[k]| * |scales[0, col]|)) / 2^45, i.e. a
+// partial sum fits as long as the scales of its own groups stay below 256 times the column's scale in group 0
+// (|q - z| <= 15, the partial's share of sum |x| <= all of it).  A partial sum of typical magnitude keeps
+// 29 bits, more than its fp32 mantissa; in general the exchange adds at most ktiles * unit / 2 to a column.
+// A partial sum that does not fit (far larger scales than group 0's, or not finite) takes the slow path: it is
+// left as fp32 in `partials` (as in the exchanges above), its K tile is marked in the column's mask word, and
+// only then the slot is bumped, with the slow-path count; the finishing thread then adds the marked partial
+// sums in K-tile order, in double.  Slots and masks live in the zeroed area that otherwise holds the arrival
+// counters (N * 16 bytes) and are left zeroed.
+constexpr int kFixedCountShift = 58;
+constexpr int kFixedSlowShift = 52;
+constexpr int kFixedBiasLog2 = 45;
+constexpr int kFixedMaxKTiles = 63;   // arrivals must fit six bits, K tiles the 64-bit mask
+
+struct FixedUnit {
+    float unit, inv_unit;  // powers of two
+};
+
+// `ref` = sum |x| * |scales[0, col]| >= 0 (or NaN / Inf, which take the largest unit).
+__device__ __forceinline__ FixedUnit fixed_unit_of(float ref) {
+    int e = static_cast<int>((__float_as_uint(ref) >> 23) & 0xffu);  // ref < 2^(e - 126)
+    e = e < 33 ? 33 : (e > 254 ? 254 : e);
+    // 2^45 units = 2^(e - 126) * 16 * 256
+    FixedUnit u;
+    u.unit = __uint_as_float(static_cast<uint32_t>(e - 32) << 23);
+    u.inv_unit = __uint_as_float(static_cast<uint32_t>(286 - e) << 23);
+    return u;
+}
+
+// Called by the threads that own a column (tid < 256), more than one K tile.  `slots` is the zeroed area.
+__device__ __forceinline__ void splitk_exchange_store_fixed(float psum, FixedUnit u, int N, int ct, int kt, int ktiles,
+                                                            unsigned long long* __restrict__ slots,
+                                                            float* __restrict__ partials,
+                                                            uint16_t* __restrict__ y) {
+    const int col = ct * kTileCols + static_cast<int>(threadIdx.x);
+    if (col >= N) return;
+    unsigned long long* slot = slots + col;
+    unsigned long long* mask = slots + N + col;
+    const float t = psum * u.inv_unit;  // exact: a power of two, and what underflows is below the unit
+    const bool fits = __builtin_fabsf(t) < 0x1p45f;  // false for NaN and for a product that overflowed
+    // t = hi * 2^24 + lo with |hi| < 2^21 and |lo| <= 2^23, both integers after rounding (garbage, unused, if !fits)
+    const float hi = __builtin_rintf(t * 0x1p-24f);
+    const float lo = __builtin_fmaf(hi, -0x1p24f, t);  // exact
+    const long long v = (static_cast<long long>(static_cast<int>(hi)) << 24) +
+                        static_cast<long long>(static_cast<int>(__builtin_rintf(lo)));
+    unsigned long long add = (1ull << kFixedCountShift) + static_cast<unsigned long long>(v + (1ll << kFixedBiasLog2));
+    if (__builtin_expect(!fits, 0)) {
+        store_agent(partials + static_cast<size_t>(kt) * N + col, psum);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        // returning, so that the wait below covers it: the mark is in memory before the slot moves
+        const unsigned long long seen = __hip_atomic_fetch_or(mask, 1ull << kt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("" ::"v"(seen));
+        __builtin_amdgcn_s_waitcnt(0);
+        add = (1ull << kFixedCountShift) + (1ull << kFixedSlowShift) + (1ull << kFixedBiasLog2);
+    }
+    const unsigned long long old = __hip_atomic_fetch_add(slot, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((old >> kFixedCountShift) != static_cast<unsigned long long>(ktiles - 1)) return;
+    const unsigned long long total = old + add;
+    const long long value = static_cast<long long>(total & ((1ull << kFixedSlowShift) - 1)) -
+                            static_cast<long long>(ktiles) * (1ll << kFixedBiasLog2);
+    double sum = static_cast<double>(value) * static_cast<double>(u.unit);
+    if (__builtin_expect(((total >> kFixedSlowShift) & 63ull) != 0, 0)) {
+        const unsigned long long m = __hip_atomic_load(mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int tt = 0; tt < ktiles; tt++) {
+            if ((m >> tt) & 1ull) sum += static_cast<double>(load_agent(partials + static_cast<size_t>(tt) * N + col));
+        }
+        __hip_atomic_store(mask, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    store_result(y + col, f32_to_bf16(static_cast<float>(sum)));
+    __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // The per-wave exchange for ROWS activation rows (M <= ROWS of them live) of a workgroup of 256 threads:
 // partial sums laid out [K tile][M][N] as in splitk_exchange_sum, one arrival counter per wave of 64 columns,
 // the last wave of a quarter reads every row of its columns back, K tiles in order (the order of
@@ -313,6 +407,7 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_wave_rows(const float (&
     uint32_t prev = 0;
     if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
+    compiler_fence();  // the read-back below stays behind the counter's return
     if (prev != static_cast<uint32_t>(ktiles - 1)) return false;
 
     // last of its quarter: every other wave's partial sums were acknowledged before its increment
@@ -401,6 +496,7 @@ __device__ __forceinline__ bool splitk_exchange_sum_per_head(float psum, float* 
     uint32_t prev = 0;
     if (tid % kWave == 0) prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     prev = __builtin_amdgcn_readfirstlane(prev);
+    compiler_fence();  // the read-back below stays behind the counter's return
     if (prev != static_cast<uint32_t>(2 * ktiles - 1)) return false;
 
     // last of its head: every other wave's partial sums were acknowledged before its increment
@@ -462,6 +558,7 @@ __device__ __forceinline__ bool splitk_exchange_sum_wide(const float (&psum)[ROW
     }
     __syncthreads();
     if (*s_prev != static_cast<uint32_t>(ktiles - 1)) return false;
+    compiler_fence();  // the read-back below stays behind the counter's return
     before_read_back();
 
     constexpr int HALF = ROWS / 2;   // rows per thread

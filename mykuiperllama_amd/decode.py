@@ -150,7 +150,9 @@ class DecodeModel:
 
         fused=False       every operator a launch of its own (ten per layer)
         fused="prologue"  the small operators inside the GEMV launches, arithmetic unchanged: bit for bit
-                          the result of fused=False
+                          the result of fused=False when that step's plain GEMVs add their K tiles in the
+                          same order (capi.set_awq_kernel_policy(1)); the product's plain GEMV adds them
+                          exactly, in fixed point, and agrees to rounding
         fused=True        ("chain") additionally the residual add and the sum of squares of the RMSNorm
                           leave with the epilogue of the producing GEMV, which saves every workgroup of the
                           consuming GEMV a pass over the whole row; the sum is added in another order, so

@@ -7,7 +7,8 @@ namespace kernel {
 
 CudaConfig::~CudaConfig() {
     if (stream_ != nullptr) {
-        // what the matmul wrapper keeps for this stream goes with it: a later stream may get the same handle
+        // what the matmul wrapper keeps for this stream goes with it (a later stream may get the same handle);
+        // the release waits for the launches still queued on the stream
         matmul_release_workspace(stream_);
         hipError_t err = hipStreamDestroy(stream_);
         if (err != hipSuccess) {

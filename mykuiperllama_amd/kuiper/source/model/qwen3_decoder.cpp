@@ -141,7 +141,8 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
 
     const int32_t big_k = std::max(std::max(c.hidden, c.intermediate), c.n_q_heads * c.head_dim);
     const int32_t big_n = std::max(std::max(c.qkv_out(), 2 * c.intermediate), c.hidden);
-    const size_t gemv_bytes = std::max<size_t>(kx_gemv_workspace_bytes(1, big_k, big_n), 262144);
+    const size_t gemv_bytes = kx_gemv_workspace_bytes(1, big_k, big_n);
+    CHECK_GT(gemv_bytes, 0u);
     gemv_workspace_ = device_bytes(gemv_bytes);
     CHECK_EQ(kx_workspace_init(gemv_workspace_.ptr<uint8_t>(), gemv_bytes, stream()), KX_OK);
     const size_t attn_bytes = kx_attn_decode_workspace_bytes(c.n_q_heads, c.head_dim, max_positions);

@@ -32,7 +32,18 @@ bool stream_is_capturing(void* stream) {
     return status != hipStreamCaptureStatusNone;
 }
 
+// The C ABI's structs carry no size field: a library built from another version of kx_hip.h would read other
+// fields, so the first call through this file compares versions.
+void check_abi_once() {
+    static const bool checked = [] {
+        CHECK_EQ(kx_abi_version(), KX_ABI_VERSION) << "libkx_hip.so and this build of the host API disagree about kx_hip.h";
+        return true;
+    }();
+    (void)checked;
+}
+
 void* workspace_for(void* stream, size_t bytes) {
+    check_abi_once();
     if (bytes == 0) {
         return nullptr;
     }
@@ -73,7 +84,24 @@ void matmul_release_workspaces() {
 }
 
 void matmul_release_workspace(void* stream) {
-    workspaces().erase(stream);
+    auto it = workspaces().find(stream);
+    if (it == workspaces().end()) return;
+    // The allocator hands a released block to the next request at once, and that request zeroes its counters:
+    // launches still queued on this stream must have finished with the block before it goes back.  A stream
+    // that records a graph cannot be waited for; its block stays in the table until matmul_release_workspaces().
+    if (stream_is_capturing(stream)) {
+        LOG(ERROR) << "the matmul workspace of a capturing stream is kept until matmul_release_workspaces()";
+        return;
+    }
+    if (it->second.buffer != nullptr) {
+        const hipError_t err = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+        if (err != hipSuccess) {
+            (void)hipGetLastError();
+            LOG(ERROR) << "could not wait for the stream before releasing its matmul workspace: "
+                       << hipGetErrorString(err);
+        }
+    }
+    workspaces().erase(it);
 }
 
 void matmul_reserve_workspace(void* stream, int32_t M, int32_t K, int32_t N) {

@@ -312,3 +312,41 @@ TEST_GPU(test_matmul, capture_without_a_reserved_workspace_is_refused_and_with_o
     ASSERT_EQ(hipGraphExecDestroy(exec), hipSuccess);
     ASSERT_EQ(hipGraphDestroy(graph), hipSuccess);
 }
+
+TEST_GPU(test_matmul, replacing_the_stream_waits_for_the_launches_that_use_its_workspace) {
+    // CudaConfig::set_stream releases the old stream's split-K workspace; the pooled allocator hands that block to
+    // the next stream's workspace at once, whose initialisation zeroes the counters.  The release therefore has
+    // to wait for the GEMVs still queued on the old stream: both results must be the oracle's.
+    AwqProblem p = make_problem(1, 12288, 4096, 128, 31415);
+    op::MatmulLayer layer(base::DeviceType::DeviceCUDA, p.N, p.K, true, p.G);
+    tensor::Tensor qw = host_tensor(base::DataType::DataTypeInt32, {p.K, p.N / 8}, p.qweight);
+    tensor::Tensor qz = host_tensor(base::DataType::DataTypeInt32, {p.K / p.G, p.N / 8}, p.qzeros);
+    tensor::Tensor sc = host_tensor(base::DataType::DataTypeFp16, {p.K / p.G, p.N}, p.scales);
+    tensor::Tensor x = host_tensor(base::DataType::DataTypeBf16, {p.M, p.K}, p.x);
+    std::vector<uint16_t> out_a(size_t(p.M) * p.N, 0x7FC0), out_b(size_t(p.M) * p.N, 0x7FC0);
+    tensor::Tensor ya = host_tensor(base::DataType::DataTypeBf16, {p.M, p.N}, out_a);
+    tensor::Tensor yb = host_tensor(base::DataType::DataTypeBf16, {p.M, p.N}, out_b);
+    for (tensor::Tensor* t : {&qw, &qz, &sc, &x, &ya, &yb}) t->to_cuda();
+    auto config = std::make_shared<kernel::CudaConfig>();
+    config->create();
+    layer.set_cuda_config(config);
+    ASSERT_TRUE(bool(layer.set_weight(0, qw)));
+    ASSERT_TRUE(bool(layer.set_weight(1, qz)));
+    layer.set_awq_scales(sc);
+    hipStream_t first = config->stream();
+    for (int i = 0; i < 40; i++) ASSERT_TRUE(bool(layer.forward(x, ya)));  // a queue of launches on the first stream
+    hipStream_t second = nullptr;
+    ASSERT_EQ(hipStreamCreate(&second), hipSuccess);
+    config->set_stream(second);  // the config owns `second` from here on
+    ASSERT_TRUE(bool(layer.forward(x, yb)));
+    ASSERT_EQ(hipStreamSynchronize(second), hipSuccess);
+    ASSERT_EQ(hipStreamSynchronize(first), hipSuccess);
+    ya.to_cpu();
+    yb.to_cpu();
+    std::memcpy(out_a.data(), ya.ptr<uint16_t>(), out_a.size() * 2);
+    std::memcpy(out_b.data(), yb.ptr<uint16_t>(), out_b.size() * 2);
+    const std::vector<double> ref = oracle_awq(p);
+    expect_close(out_a, ref);
+    expect_close(out_b, ref);
+    ASSERT_EQ(hipStreamDestroy(first), hipSuccess);
+}

@@ -59,11 +59,11 @@ def check_against_oracle(oracle, p, y_bits):
 SHAPES_8B = sorted(set(synth.QWEN3_8B.values()))
 
 
-@pytest.fixture(params=["by_shape", "vector", "mfma", "stream", "wide"], autouse=True)
+@pytest.fixture(params=["by_shape", "vector", "mfma"], autouse=True)
 def kernel_policy(request, capi):
-    """Every test in this file runs under each kernel policy: the product's choice, either product kernel
-    forced, and the two measured alternatives that the internal entry point keeps selectable."""
-    capi.set_awq_kernel_policy({"by_shape": 0, "vector": 1, "mfma": 2, "stream": 3, "wide": 4}[request.param])
+    """Every test in this file runs under each kernel policy: the product's choice and either product kernel
+    forced through the internal entry point."""
+    capi.set_awq_kernel_policy({"by_shape": 0, "vector": 1, "mfma": 2}[request.param])
     yield request.param
     capi.set_awq_kernel_policy(0)
 

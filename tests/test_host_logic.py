@@ -67,7 +67,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_error_strings(lib):
-    assert lib.kx_abi_version() >= 2
+    assert lib.kx_abi_version() == 3  # KX_ABI_VERSION of include/kx_hip.h
     assert lib.kx_error_string(0) == b"ok"
     for code in (-1, -2, -3, -4):
         assert len(lib.kx_error_string(code)) > 5

@@ -40,7 +40,7 @@ def _both(capi, torch, name, M, K, N):
 
 def test_static_scratch_entry_point_matches_the_workspace_entry_point(capi, torch, oracle):
     print("no-alloc entry point: 12288x4096 M=1, then 1024x512 M=2, then 4096x12288 M=3", flush=True)
-    assert capi.load().kx_gemv_awq_static_scratch_bytes() == 262144 + (8 << 20)
+    assert capi.load().kx_gemv_awq_static_scratch_bytes() == 524288 + (8 << 20)
     # two calls in a row on the shared array, the second one smaller, a third one on the MFMA kernel
     for name, M, K, N in (("static_a", 1, 12288, 4096), ("static_b", 2, 1024, 512), ("static_c", 3, 4096, 12288)):
         p, want, got = _both(capi, torch, name, M, K, N)
@@ -67,5 +67,8 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(capi, torch):
     assert L.kx_gemv_awq_bf16_static(*args, M, K, N, 128, s) == -3
     assert L.kx_gemv_awq_bf16_static(None, *args[1:], 1, K, N, 128, s) == -1
     assert L.kx_gemv_awq_bf16_static(*args, 1, K, N, 100, s) == -2
+    assert L.kx_gemv_awq_bf16_static(args[0] + 2, *args[1:], 1, K, N, 128, s) == -4  # x not 16-byte aligned
+    # the fused 8B shapes at several rows are past the array as well: gate|up 4096 -> 24576 at four rows
+    assert capi.workspace_bytes(4, 4096, 24576) > L.kx_gemv_awq_static_scratch_bytes()
     torch.cuda.synchronize()
     assert bool((y == 7.0).all())  # nothing was launched
