@@ -3,8 +3,10 @@
 //
 // Per KV head the first stage leaves, for every chunk c of the context and each of its G query heads:
 //   part_out[kvh][c][g][0..127]   the unnormalised weighted sum of V rows, relative to the chunk maximum
-//   part_ml [kvh][c][g][0..1]     the chunk maximum m_c and the chunk sum of exponentials l_c (0: empty chunk)
-// The merged head is  sum_c part_out[c] * f_c / sum_c l_c * f_c  with  f_c = exp(m_c - max_c m_c).
+//   part_ml [kvh][c][g][0..1]     the chunk maximum m_c of the scores in units of log 2 (score * log2 e) and the
+//                                 chunk sum of exponentials l_c (0: empty chunk)
+// The merged head is  sum_c part_out[c] * f_c / sum_c l_c * f_c  with  f_c = 2^(m_c - max_c m_c), the hardware's
+// exponential (v_exp_f32) like the first stage's.
 #ifndef KX_ATTN_MERGE_H
 #define KX_ATTN_MERGE_H
 
@@ -76,7 +78,7 @@ __device__ __forceinline__ float attn_merge_finish(const MergeStats<PER_LANE>& s
 #pragma unroll
     for (int u = 0; u < PER_LANE; u++) {
         const int c = lane + u * kWave;
-        const float f = st.l[u] > 0.0f ? expf(st.m[u] - m) : 0.0f;  // chunks past the context have l == 0
+        const float f = st.l[u] > 0.0f ? __builtin_amdgcn_exp2f(st.m[u] - m) : 0.0f;  // chunks past the context have l == 0
         if (c < kMergeParts * per_part) s_factor[attn_factor_slot(c, per_part)] = f;
         l += st.l[u] * f;
     }

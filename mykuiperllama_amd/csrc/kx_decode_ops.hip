@@ -148,11 +148,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // Scores, then softmax weights, per head; rows padded so that the sixteen-byte reads of the
     // second pass (one row per lane) do not all start on the same bank.
     __shared__ __attribute__((aligned(16))) float s_score[kMaxGroup][CHUNK + 4];
-    // The chunk's V rows, row-major, one dword of padding per row: the second pass reads them
-    // transposed (eight positions of one dim per lane), and with 65 dwords per row the four blocks of
-    // eight positions that a read instruction touches fall on different banks.
-    constexpr int kVRow = kHeadDim / 2 + 1;
-    __shared__ uint32_t s_v[CHUNK][kVRow];
+    // The chunk's V rows, row-major, two dwords of padding per row: the second pass reads a dword (two
+    // neighbouring dims) of eight positions per lane, and with 66 dwords per row the four blocks of eight
+    // positions that a read instruction touches fall on different banks.
+    constexpr int kVRow = kHeadDim / 2 + 2;
+    __shared__ __attribute__((aligned(8))) uint32_t s_v[CHUNK][kVRow];
 
     const int kvh = blockIdx.y;
     const int chunk = blockIdx.x;
@@ -225,7 +225,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // for *pos and the round trip for the rows one after the other.  Such a chunk runs through with
     // everything masked and reports max = -inf, sum = 0.
 
-    // pass 1: scores
+    // pass 1: scores, in units of log 2 (the exponentials below and in the merge are the hardware's exp2)
+    const float scale2 = scale * 1.44269504088896341f;
     const bool q_live = mc < G;
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
@@ -242,10 +243,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             // rows past G exist in s_score and nobody reads them: no test, no branch around the store
-            s_score[4 * mb + v][pl] = (p0 + pl < ctx) ? d[v] * scale : -INFINITY;
+            s_score[4 * mb + v][pl] = (p0 + pl < ctx) ? d[v] * scale2 : -INFINITY;
         }
     }
-    __syncthreads();
+    // LDS only: the V rows stay in flight, and the statistics below run while they arrive (a full
+    // __syncthreads() would make the scores wait for every V row)
+    lds_barrier();
 
     // softmax statistics per head over the chunk; wave w serves heads w, w + 4, ...
     for (int g = tid / kWave; g < G; g += kAttnThreads / kWave) {
@@ -263,7 +266,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
         float l = 0.0f;
 #pragma unroll
         for (int u = 0; u < PER_LANE; u++) {
-            sc[u] = expf(sc[u] - shift);
+            sc[u] = __builtin_amdgcn_exp2f(sc[u] - shift);
             l += sc[u];
             s_score[g][lane + u * kWave] = sc[u];
         }
@@ -278,88 +281,88 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
             }
         }
     }
-    // The V rows go to LDS while the statistics are being taken: rows past the context carry weight 0,
-    // their (arbitrary) contents are zeroed so that a stray NaN or infinity cannot leak through 0 * x.
-#pragma unroll
-    for (int it = 0; it < ITERS; it++) {
-        const int pl = it * 16 + slot;
-        const bool live = p0 + pl < ctx;
-        uint32_t* dst = &s_v[pl][4 * sub];
-        dst[0] = live ? vraw[it].x : 0u;
-        dst[1] = live ? vraw[it].y : 0u;
-        dst[2] = live ? vraw[it].z : 0u;
-        dst[3] = live ? vraw[it].w : 0u;
-    }
-    __syncthreads();
 
-    // pass 2: weighted sum of V rows on the matrix cores, D[head][dim] = sum over the chunk's
-    // positions in steps of 32, A = the softmax weights (row = head), B = the V rows (column = dim).
-    // Lane (mc, mb) supplies positions 32 s + 8 mb .. + 7 of head mc and of dim mc of the tile.  The
-    // weights are fp32 and the operands bf16: a weight enters as its bf16 rounding plus the bf16
-    // rounding of what that left over, two MFMAs per step (error 2^-17 relative instead of 2^-9).
-    // A wave takes two of the eight sixteen-dim tiles; nothing is left to add up across threads.
+    // pass 2, in two halves of the chunk: the V rows of a half go to LDS (rows past the context carry weight 0,
+    // their arbitrary contents are zeroed so that a stray NaN or infinity cannot leak through 0 * x), a barrier,
+    // and the half's weighted sum of V rows on the matrix cores, D[head][dim] = sum over the half's positions in
+    // steps of 32, A = the softmax weights (row = head), B = the V rows (column = dim).  The first half is summed
+    // while the rows of the second are still arriving (loads return in order), so that only the second half's
+    // chain stands behind the last byte.
+    // Lane (mc, mb) supplies positions 32 s + 8 mb .. + 7 of head mc and of one dim.  A wave takes 32 dims as two
+    // tiles, the even dims and the odd ones, so that one dword read per position feeds both.  The weights are
+    // fp32 and the operands bf16: a weight enters as its bf16 rounding plus the bf16 rounding of what that left
+    // over, two MFMAs per step (error 2^-17 relative instead of 2^-9).
     constexpr int KSTEPS = CHUNK / 32;
-    const uint16_t* sv16 = reinterpret_cast<const uint16_t*>(&s_v[0][0]);
+    static_assert(ITERS % 2 == 0 && KSTEPS % 2 == 0, "two halves of whole steps");
     f32x4v dacc[2];
     dacc[0] = dacc[1] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-        const float4* prow = reinterpret_cast<const float4*>(&s_score[q_head][32 * ks + 8 * mb]);
-        const float4 pa = prow[0];
-        const float4 pb = prow[1];
-        const float pw[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
-        uint32_t hi[4], lo[4];
+    for (int half = 0; half < 2; half++) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float w0 = q_live ? pw[2 * j] : 0.0f;
-            const float w1 = q_live ? pw[2 * j + 1] : 0.0f;
-            hi[j] = f32x2_to_bf16x2(w0, w1);
-            lo[j] = f32x2_to_bf16x2(w0 - __uint_as_float(hi[j] << 16), w1 - __uint_as_float(hi[j] & 0xffff0000u));
+        for (int i = 0; i < ITERS / 2; i++) {
+            const int it = half * (ITERS / 2) + i;
+            const int pl = it * 16 + slot;
+            const bool live = p0 + pl < ctx;
+            u32x2* dst = reinterpret_cast<u32x2*>(&s_v[pl][4 * sub]);
+            dst[0] = u32x2{live ? vraw[it].x : 0u, live ? vraw[it].y : 0u};
+            dst[1] = u32x2{live ? vraw[it].z : 0u, live ? vraw[it].w : 0u};
         }
-        const bf16x8 a_hi = as_bf16x8(hi[0], hi[1], hi[2], hi[3]);
-        const bf16x8 a_lo = as_bf16x8(lo[0], lo[1], lo[2], lo[3]);
+        lds_barrier();  // the first one also publishes the weights
 #pragma unroll
-        for (int n = 0; n < 2; n++) {
-            const int col = 16 * (2 * wave + n) + mc;  // dim
-            const uint16_t* vcol = sv16 + static_cast<size_t>(32 * ks + 8 * mb) * (2 * kVRow) + col;
-            uint32_t vw[4];
+        for (int k = 0; k < KSTEPS / 2; k++) {
+            const int ks = half * (KSTEPS / 2) + k;
+            const float4* prow = reinterpret_cast<const float4*>(&s_score[q_head][32 * ks + 8 * mb]);
+            const float4 pa = prow[0];
+            const float4 pb = prow[1];
+            const float pw[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
+            uint32_t hi[4], lo[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const uint32_t even = vcol[(2 * j) * (2 * kVRow)];
-                const uint32_t odd = vcol[(2 * j + 1) * (2 * kVRow)];
-                vw[j] = even | (odd << 16);
+                const float w0 = q_live ? pw[2 * j] : 0.0f;
+                const float w1 = q_live ? pw[2 * j + 1] : 0.0f;
+                hi[j] = f32x2_to_bf16x2(w0, w1);
+                lo[j] = f32x2_to_bf16x2(w0 - __uint_as_float(hi[j] << 16), w1 - __uint_as_float(hi[j] & 0xffff0000u));
             }
-            const bf16x8 b_op = as_bf16x8(vw[0], vw[1], vw[2], vw[3]);
-            dacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_op, dacc[n], 0, 0, 0);
-            dacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b_op, dacc[n], 0, 0, 0);
+            const bf16x8 a_hi = as_bf16x8(hi[0], hi[1], hi[2], hi[3]);
+            const bf16x8 a_lo = as_bf16x8(lo[0], lo[1], lo[2], lo[3]);
+            // dims 32 wave + 2 mc (low half of the dword) and + 1 (high half) of eight positions
+            uint32_t vd[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) vd[j] = s_v[32 * ks + 8 * mb + j][16 * wave + mc];
+            uint32_t even[4], odd[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                even[j] = __builtin_amdgcn_perm(vd[2 * j + 1], vd[2 * j], 0x05040100u);  // low halves of two positions
+                odd[j] = __builtin_amdgcn_perm(vd[2 * j + 1], vd[2 * j], 0x07060302u);   // high halves
+            }
+            const bf16x8 b_even = as_bf16x8(even[0], even[1], even[2], even[3]);
+            const bf16x8 b_odd = as_bf16x8(odd[0], odd[1], odd[2], odd[3]);
+            dacc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_even, dacc[0], 0, 0, 0);
+            dacc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_odd, dacc[1], 0, 0, 0);
+            dacc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b_even, dacc[0], 0, 0, 0);
+            dacc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b_odd, dacc[1], 0, 0, 0);
         }
     }
-    // the lane holds heads 4 mb .. 4 mb + 3 of dim `col`
-    // One test on the kind of store and one on the lane's heads around all eight stores: inside the loops they
+    // The lane holds heads 4 mb .. 4 mb + 3 of dims 32 wave + 2 mc and + 1: one eight-byte store per head.
+    // One test on the kind of store and one on the lane's heads around all four stores: inside the loop they
     // had become two branches per store.  (A lane's four heads are all live or all past G when G is a multiple
     // of four; other groupings take the per-head test.)
     const bool all_four = 4 * mb + 3 < G;
+    const int dim0 = 32 * wave + 2 * mc;
     if (one_sequence && all_four) {
 #pragma unroll
-        for (int n = 0; n < 2; n++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                store_result(out_base + (4 * mb + v) * kHeadDim + 16 * (2 * wave + n) + mc, dacc[n][v]);
-            }
-        }
-    } else if (all_four) {
-#pragma unroll
-        for (int n = 0; n < 2; n++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) out_base[(4 * mb + v) * kHeadDim + 16 * (2 * wave + n) + mc] = dacc[n][v];
+        for (int v = 0; v < 4; v++) {
+            const u32x2 pair = {__float_as_uint(dacc[0][v]), __float_as_uint(dacc[1][v])};
+            unsigned long long bits;
+            __builtin_memcpy(&bits, &pair, 8);
+            store_result(reinterpret_cast<unsigned long long*>(out_base + (4 * mb + v) * kHeadDim + dim0), bits);
         }
     } else {
 #pragma unroll
-        for (int n = 0; n < 2; n++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int head = 4 * mb + v;
-                if (head < G) out_base[head * kHeadDim + 16 * (2 * wave + n) + mc] = dacc[n][v];
+        for (int v = 0; v < 4; v++) {
+            const int head = 4 * mb + v;
+            if (all_four || head < G) {
+                *reinterpret_cast<float2*>(out_base + head * kHeadDim + dim0) = make_float2(dacc[0][v], dacc[1][v]);
             }
         }
     }
