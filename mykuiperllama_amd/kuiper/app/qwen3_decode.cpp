@@ -1,5 +1,5 @@
-// kx_qwen3_decode [--graph] [--layers] [--max-positions N] [--generate N] file.safetensors token [token ...]
-// kx_qwen3_decode [--graph] [--layers] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]
+// kx_qwen3_decode [--graph] [--layers | --operators] [--max-positions N] [--generate N] file.safetensors token [token ...]
+// kx_qwen3_decode [--graph] [--layers | --operators] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]
 //
 // First form: feeds the tokens one by one to model::Qwen3Decoder from an empty KV cache (token i at
 // position i) and prints one line per step:
@@ -9,9 +9,10 @@
 // Second form: random-init weights of the named architecture, caches filled with N(0,1) up to the
 // context length, then S steps at position C timed back to back; prints one JSON line with
 // ms_per_step and tokens_per_s (batch 1, lm_head and argmax included).
-// With --graph the step is captured in a HIP graph first and every step replays it.  With --layers the
-// step is one kuiper layer forward() per operator (ten launches per decoder layer) instead of the
-// fused entry points.
+// With --graph the step is captured in a HIP graph first and every step replays it.  With --layers every
+// launch of the step is the forward() of a kuiper layer, the projections in their fused form (the same five or
+// six launches per decoder layer as the fused entry points called directly); with --operators the step is one
+// kuiper layer forward() per operator (ten launches per decoder layer).
 #include <cinttypes>
 #include <cstdio>
 #include <cstdlib>
@@ -23,7 +24,12 @@
 
 namespace {
 
-int run_random(const std::string& name, int32_t context, int32_t steps, int32_t warmup, bool graph, bool layers) {
+const char* path_name(model::DecodePath p) {
+    return p == model::DecodePath::Layers ? "layers" : (p == model::DecodePath::Operators ? "operators" : "fused");
+}
+
+int run_random(const std::string& name, int32_t context, int32_t steps, int32_t warmup, bool graph,
+               model::DecodePath decode_path) {
     model::Qwen3Config c;
     if (name == "qwen3-8b") {
         c.layers = 36, c.hidden = 4096, c.intermediate = 12288, c.n_q_heads = 32, c.n_kv_heads = 8, c.vocab = 151936;
@@ -39,7 +45,7 @@ int run_random(const std::string& name, int32_t context, int32_t steps, int32_t 
         std::fprintf(stderr, "--context C (>= 0), --steps S (>= 1) and --warmup W (>= 0) are needed with --random\n");
         return 2;
     }
-    model::Qwen3Decoder decoder(c, context + 1, layers ? model::DecodePath::Layers : model::DecodePath::Fused);
+    model::Qwen3Decoder decoder(c, context + 1, decode_path);
     decoder.init_random(20251125);
     decoder.fill_cache_random(context, 7);
     base::Status st = graph ? decoder.capture() : base::error::success();
@@ -52,7 +58,7 @@ int run_random(const std::string& name, int32_t context, int32_t steps, int32_t 
     std::printf("{\"model\": \"%s\", \"weights\": \"random-init\", \"context\": %d, \"graph\": %s, \"path\": \"%s\", "
                 "\"launches_per_step\": %d, \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
                 "\"tokens_per_s\": %.2f}\n",
-                name.c_str(), context, graph ? "true" : "false", layers ? "layers" : "fused", decoder.launches_per_step(), steps,
+                name.c_str(), context, graph ? "true" : "false", path_name(decode_path), decoder.launches_per_step(), steps,
                 warmup, ms,
                 1000.0 / ms);
     return 0;
@@ -61,7 +67,8 @@ int run_random(const std::string& name, int32_t context, int32_t steps, int32_t 
 }  // namespace
 
 int main(int argc, char** argv) {
-    bool graph = false, layers = false;
+    bool graph = false;
+    model::DecodePath decode_path = model::DecodePath::Fused;
     int32_t max_positions = 0, context = -1, steps = 50, warmup = 10, generate = 0;
     std::string path, random_model;
     std::vector<int32_t> tokens;
@@ -70,7 +77,9 @@ int main(int argc, char** argv) {
         if (std::strcmp(argv[i], "--graph") == 0) {
             graph = true;
         } else if (std::strcmp(argv[i], "--layers") == 0) {
-            layers = true;
+            decode_path = model::DecodePath::Layers;
+        } else if (std::strcmp(argv[i], "--operators") == 0) {
+            decode_path = model::DecodePath::Operators;
         } else if (std::strcmp(argv[i], "--max-positions") == 0 && i + 1 < argc) {
             max_positions = number(i);
         } else if (std::strcmp(argv[i], "--generate") == 0 && i + 1 < argc) {
@@ -89,11 +98,11 @@ int main(int argc, char** argv) {
             tokens.push_back(static_cast<int32_t>(std::strtol(argv[i], nullptr, 10)));
         }
     }
-    if (!random_model.empty()) return run_random(random_model, context, steps, warmup, graph, layers);
+    if (!random_model.empty()) return run_random(random_model, context, steps, warmup, graph, decode_path);
     if (path.empty() || tokens.empty()) {
         std::fprintf(stderr,
-                     "usage: %s [--graph] [--layers] [--max-positions N] [--generate N] file.safetensors token [token ...]\n"
-                     "       %s [--graph] [--layers] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]\n",
+                     "usage: %s [--graph] [--layers | --operators] [--max-positions N] [--generate N] file.safetensors token [token ...]\n"
+                     "       %s [--graph] [--layers | --operators] --random qwen3-8b|qwen3-32b|tiny --context C [--steps S] [--warmup W]\n",
                      argv[0], argv[0]);
         return 2;
     }
@@ -116,7 +125,7 @@ int main(int argc, char** argv) {
     std::fprintf(stderr, "layers %d hidden %d intermediate %d q heads %d kv heads %d vocab %d group %d\n", config.layers,
                  config.hidden, config.intermediate, config.n_q_heads, config.n_kv_heads, config.vocab,
                  config.group_size);
-    model::Qwen3Decoder decoder(config, max_positions, layers ? model::DecodePath::Layers : model::DecodePath::Fused);
+    model::Qwen3Decoder decoder(config, max_positions, decode_path);
     st = decoder.load(file);
     if (st && graph) st = decoder.capture();
     if (!st) {

@@ -57,12 +57,16 @@ struct Qwen3Config {
 };
 
 // How a step is put together.
-//   Fused   the fused entry points of kx_hip.h, five or six launches per decoder layer (the fast path)
-//   Layers  one kuiper layer per operator, forward() by forward() — EmbeddingLayer, RmsNormLayer (with
-//           the residual add in front), MatmulLayer, RoPELayer, MultiHeadAttention, SwiGLULayer — ten
-//           launches per decoder layer: what a model written against the layer API of
-//           kuiper/include/op/layer.h looks like, and the yardstick the fused path is held against
-enum class DecodePath { Fused, Layers };
+//   Fused      the fused entry points of kx_hip.h called directly, five or six launches per decoder layer
+//   Layers     the same launches through the layer API of kuiper/include/op/layer.h: every launch is the
+//              forward() of a kuiper layer — EmbeddingLayer, RmsNormLayer (first layer's input and the final norm),
+//              MultiHeadAttention (its first stage), and four MatmulLayers per decoder layer whose fused form
+//              (MatmulLayer::set_fusion) carries the norms, the rotation, the merge, SwiGLU and the residual add
+//   Operators  one kuiper layer per operator, forward() by forward() — EmbeddingLayer, RmsNormLayer (with
+//              the residual add in front), MatmulLayer, RoPELayer, MultiHeadAttention, SwiGLULayer — ten
+//              launches per decoder layer: a model that uses the layer API without the fused forms, and the
+//              yardstick the other two are held against
+enum class DecodePath { Fused, Layers, Operators };
 
 class Qwen3Decoder {
 public:
@@ -121,7 +125,8 @@ private:
     int enqueue_step();  // 0 or the first failing entry point's return code
     int enqueue_step_fused();
     int enqueue_step_layers();
-    void attach_layer_weights();  // Layers path: gains and tables into the operator layers
+    int enqueue_step_operators();
+    void attach_layer_weights();  // Layers and Operators paths: gains and tables into the layers, fused forms set
 
     Qwen3Config config_;
     int32_t max_positions_ = 0;
@@ -133,7 +138,7 @@ private:
     tensor::Tensor embed_, final_norm_;
     std::unique_ptr<op::MatmulLayer> lm_head_;
     tensor::Tensor x_, h_, q_, attn_, gate_up_, logits_, sumsq_;
-    // Layers path only
+    // Layers and Operators paths
     std::vector<LayerOps> layer_ops_;
     std::unique_ptr<op::EmbeddingLayer> embedding_op_;
     std::unique_ptr<op::MultiHeadAttention> attention_op_;

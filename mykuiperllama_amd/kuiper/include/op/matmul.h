@@ -15,11 +15,26 @@
 //
 // forward() follows the pattern of VecAddLayer::forward (kuiper/source/op/add.cpp:36-49): check(),
 // then kernel::get_matmul_kernel[_awq](device_type_)(..., stream).  No synchronisation inside.
+//
+// A GPU AWQ layer can take its neighbours in a decoder layer into its launch (set_fusion): the
+// activations produced on the way in (SwiGLU of two rows, RMSNorm from the row's tile sums of squares, the
+// merge of the attention chunks) and the result consumed on the way out (residual add with the new row's
+// tile sums, or per-head norm + rotation + KV-cache append of a q|k|v row).  forward() then goes through
+// kernel::get_matmul_chain_kernel(device_type_); input 0 / output 0 are used only by the ends that stay
+// plain rows.  One activation row.  This is the quantised-layer hook the reference reserves in
+// kuiper/include/op/layer.h:122-156 (scales, group size on LayerParam), extended to the launches
+// themselves.
 #ifndef KUIPER_INCLUDE_OP_MATMUL_H
 #define KUIPER_INCLUDE_OP_MATMUL_H
 
+#include <memory>
+
 #include "base/cuda_config.h"
 #include "op/layer.h"
+
+namespace kernel {
+struct MatmulChain;
+}
 
 namespace op {
 
@@ -47,14 +62,23 @@ public:
     void set_awq_scales(const tensor::Tensor& scales);
     const tensor::Tensor& awq_scales() const;
 
+    // The fused form of this layer's launch: what kernel::MatmulChain describes (its x / y are ignored when the
+    // corresponding end is a plain row: input 0 / output 0 of the layer are used).  GPU AWQ layers only.
+    base::Status set_fusion(const kernel::MatmulChain& chain);
+    void clear_fusion();
+    bool fused() const;
+
     int32_t dim0() const;
     int32_t dim1() const;
     int32_t group_size() const;
     bool is_quant_layer() const;
 
 private:
+    base::Status forward_fused();
+
     int32_t dim0_ = 0;  // N
     int32_t dim1_ = 0;  // K
+    std::shared_ptr<kernel::MatmulChain> fusion_;
 };
 
 }  // namespace op

@@ -20,6 +20,11 @@ public:
     base::Status check() const override;
     base::Status forward() override;
     using TypedLayer::forward;
+    // GPU only: the first stage alone.  Inputs 0..3 as for forward(); the per-chunk results stay in chunks(), for
+    // a MatmulLayer whose fused launch merges them on its way in (kernel::MatmulChain::In::AttentionChunks).
+    base::Status forward_chunks(const tensor::Tensor& q, const tensor::Tensor& pos, const tensor::Tensor& k_cache,
+                                const tensor::Tensor& v_cache);
+    const tensor::Tensor& chunks() const { return workspace_; }
     // Allocates the GPU workspace for caches of max_positions rows now, so that forward() allocates
     // nothing later (a stream under graph capture must not).  No effect on a host layer.
     base::Status reserve(int32_t max_positions);

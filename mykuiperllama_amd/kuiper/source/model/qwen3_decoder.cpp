@@ -9,6 +9,7 @@
 
 #include "base/alloc.h"
 #include "kernel/hip/matmul_kernel.h"
+#include "kernel/kernel_interface.h"
 #include "kx_hip.h"
 #include "random_fill.h"
 
@@ -151,12 +152,9 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
 
     CHECK_EQ(hipHostMalloc(reinterpret_cast<void**>(&host_io_), 3 * sizeof(int32_t), hipHostMallocDefault), hipSuccess);
 
-    if (path_ == DecodePath::Layers) {
+    if (path_ != DecodePath::Fused) {
         const base::DeviceType gpu = base::DeviceType::DeviceCUDA;
-        qkv_ = device_tensor(bf16, {c.qkv_out()});
-        o_ = device_tensor(bf16, {c.hidden});
-        act_ = device_tensor(bf16, {c.intermediate});
-        down_ = device_tensor(bf16, {c.hidden});
+        const bool operators = path_ == DecodePath::Operators;
         auto borrowed = [&](base::DataType type, int32_t n, void* ptr) {
             tensor::Tensor t(type, n, false, nullptr, ptr);
             t.set_device_type(gpu);  // a borrowed buffer does not know where it lives
@@ -168,26 +166,36 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
         up_view_ = borrowed(bf16, c.intermediate, u16(gate_up_) + c.intermediate);
         embedding_op_ = std::make_unique<op::EmbeddingLayer>(gpu, c.vocab, c.hidden);
         attention_op_ = std::make_unique<op::MultiHeadAttention>(gpu, c.n_q_heads, c.n_kv_heads);
-        swiglu_op_ = std::make_unique<op::SwiGLULayer>(gpu, c.intermediate);
         final_norm_op_ = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
         embedding_op_->set_cuda_config(stream_);
         attention_op_->set_cuda_config(stream_);
-        swiglu_op_->set_cuda_config(stream_);
         final_norm_op_->set_cuda_config(stream_);
         lm_head_->set_cuda_config(stream_);
-        layer_ops_.resize(layers_.size());
-        for (size_t i = 0; i < layers_.size(); i++) {
+        if (operators) {
+            qkv_ = device_tensor(bf16, {c.qkv_out()});
+            o_ = device_tensor(bf16, {c.hidden});
+            act_ = device_tensor(bf16, {c.intermediate});
+            down_ = device_tensor(bf16, {c.hidden});
+            swiglu_op_ = std::make_unique<op::SwiGLULayer>(gpu, c.intermediate);
+            swiglu_op_->set_cuda_config(stream_);
+        }
+        // the fused path needs one stand-alone norm: the embedding row comes without its tile sums
+        layer_ops_.resize(operators ? layers_.size() : 1);
+        for (size_t i = 0; i < layer_ops_.size(); i++) {
             LayerOps& ops = layer_ops_[i];
             ops.input_norm = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
+            ops.input_norm->set_cuda_config(stream_);
+            if (!operators) continue;
             ops.post_norm = std::make_unique<op::RmsNormLayer>(gpu, c.hidden, c.rms_eps);
             ops.rope = std::make_unique<op::RoPELayer>(gpu, c.n_q_heads, c.n_kv_heads, c.rope_theta, c.rms_eps);
-            ops.input_norm->set_cuda_config(stream_);
             ops.post_norm->set_cuda_config(stream_);
             ops.rope->set_cuda_config(stream_);
-            layers_[i].qkv->set_cuda_config(stream_);
-            layers_[i].o->set_cuda_config(stream_);
-            layers_[i].gate_up->set_cuda_config(stream_);
-            layers_[i].down->set_cuda_config(stream_);
+        }
+        for (LayerWeights& L : layers_) {
+            L.qkv->set_cuda_config(stream_);
+            L.o->set_cuda_config(stream_);
+            L.gate_up->set_cuda_config(stream_);
+            L.down->set_cuda_config(stream_);
         }
         // everything a forward() would allocate on first use, now: a captured stream must not allocate
         CHECK(attention_op_->reserve(max_positions));
@@ -198,7 +206,7 @@ Qwen3Decoder::Qwen3Decoder(const Qwen3Config& config, int32_t max_positions, Dec
 
 Qwen3Decoder::~Qwen3Decoder() {
     if (stream_) (void)hipStreamSynchronize(stream());
-    if (stream_ && path_ == DecodePath::Layers) kernel::matmul_release_workspace(stream());  // the stream goes away with us
+    if (stream_ && path_ != DecodePath::Fused) kernel::matmul_release_workspace(stream());  // the stream goes away with us
     if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_) (void)hipGraphDestroy(graph_);
     if (host_io_) (void)hipHostFree(host_io_);
@@ -246,14 +254,79 @@ base::Status Qwen3Decoder::load(const SafetensorsFile& file) {
 }
 
 void Qwen3Decoder::attach_layer_weights() {
-    if (path_ != DecodePath::Layers) return;
+    if (path_ == DecodePath::Fused) return;
     CHECK(embedding_op_->set_weight(0, embed_));
     CHECK(final_norm_op_->set_weight(0, final_norm_));
+    if (path_ == DecodePath::Operators) {
+        for (size_t i = 0; i < layers_.size(); i++) {
+            CHECK(layer_ops_[i].input_norm->set_weight(0, layers_[i].input_norm));
+            CHECK(layer_ops_[i].post_norm->set_weight(0, layers_[i].post_norm));
+            CHECK(layer_ops_[i].rope->set_weight(0, layers_[i].q_norm));
+            CHECK(layer_ops_[i].rope->set_weight(1, layers_[i].k_norm));
+        }
+        return;
+    }
+    // Layers: the fused form of every projection, set once; a step is then one forward() per launch
+    const Qwen3Config& c = config_;
+    using Chain = kernel::MatmulChain;
+    CHECK(layer_ops_[0].input_norm->set_weight(0, layers_[0].input_norm));
     for (size_t i = 0; i < layers_.size(); i++) {
-        CHECK(layer_ops_[i].input_norm->set_weight(0, layers_[i].input_norm));
-        CHECK(layer_ops_[i].post_norm->set_weight(0, layers_[i].post_norm));
-        CHECK(layer_ops_[i].rope->set_weight(0, layers_[i].q_norm));
-        CHECK(layer_ops_[i].rope->set_weight(1, layers_[i].k_norm));
+        LayerWeights& L = layers_[i];
+        Chain qkv;
+        if (i == 0) {
+            qkv.in = Chain::In::Row;  // input 0 of the layer: the row the stand-alone norm leaves in h_
+        } else {
+            qkv.in = Chain::In::NormFromTileSums;
+            qkv.norm_row = x_;
+            qkv.norm_tile_sumsq = sumsq_;
+            qkv.norm_gain = L.input_norm;
+            qkv.norm_eps = c.rms_eps;
+        }
+        qkv.out = Chain::Out::QkvRope;
+        qkv.q_gain = L.q_norm;
+        qkv.k_gain = L.k_norm;
+        qkv.q_out = q_;
+        qkv.k_cache = L.k_cache;
+        qkv.v_cache = L.v_cache;
+        qkv.pos = pos_view_;
+        qkv.rope_n_q_heads = c.n_q_heads;
+        qkv.rope_n_kv_heads = c.n_kv_heads;
+        qkv.rope_theta = c.rope_theta;
+        qkv.qk_eps = c.rms_eps;
+        CHECK(L.qkv->set_fusion(qkv));
+
+        Chain o;
+        if (merge_in_o_) {
+            o.in = Chain::In::AttentionChunks;
+            o.attention_chunks = attention_op_->chunks();  // reserved for max_positions in the constructor: it stays put
+            o.n_q_heads = c.n_q_heads;
+            o.n_kv_heads = c.n_kv_heads;
+            o.max_positions = max_positions_;
+        } else {
+            o.in = Chain::In::Row;  // input 0: the merged attention output
+        }
+        o.out = Chain::Out::Residual;
+        o.residual = x_;
+        o.tile_sumsq = sumsq_;
+        CHECK(L.o->set_fusion(o));
+
+        Chain gate_up;
+        gate_up.in = Chain::In::NormFromTileSums;
+        gate_up.norm_row = x_;
+        gate_up.norm_tile_sumsq = sumsq_;
+        gate_up.norm_gain = L.post_norm;
+        gate_up.norm_eps = c.rms_eps;
+        gate_up.out = Chain::Out::Row;  // output 0 of the layer
+        CHECK(L.gate_up->set_fusion(gate_up));
+
+        Chain down;
+        down.in = Chain::In::SwiGLU;
+        down.gate = gate_view_;
+        down.up = up_view_;
+        down.out = Chain::Out::Residual;
+        down.residual = x_;
+        down.tile_sumsq = sumsq_;
+        CHECK(L.down->set_fusion(down));
     }
 }
 
@@ -347,18 +420,23 @@ base::Status Qwen3Decoder::time_steps(int32_t token, int32_t pos, int32_t steps,
 }
 
 int32_t Qwen3Decoder::launches_per_step() const {
-    const int32_t per_layer = path_ == DecodePath::Layers ? 10 : (merge_in_o_ ? 5 : 6);
-    return 1 + config_.layers * per_layer + 3;  // embedding; layers; final norm, lm_head, argmax
+    const int32_t per_layer = path_ == DecodePath::Operators ? 10 : (merge_in_o_ ? 5 : 6);
+    // embedding; layers; final norm, lm_head, argmax; the Layers path norms the embedding row in a launch of its own
+    return 1 + config_.layers * per_layer + 3 + (path_ == DecodePath::Layers ? 1 : 0);
 }
 
 int Qwen3Decoder::enqueue_step() {
-    return path_ == DecodePath::Layers ? enqueue_step_layers() : enqueue_step_fused();
+    switch (path_) {
+        case DecodePath::Layers: return enqueue_step_layers();
+        case DecodePath::Operators: return enqueue_step_operators();
+        default: return enqueue_step_fused();
+    }
 }
 
 // One forward() per operator, in the order of the model's formulas.  A layer reports a refused
 // tensor through its Status; a failed launch aborts inside the layer's kernel wrapper, as in the
 // reference's GPU wrappers.
-int Qwen3Decoder::enqueue_step_layers() {
+int Qwen3Decoder::enqueue_step_operators() {
     const Qwen3Config& c = config_;
 #define KX_LAYER(call)                          \
     do {                                        \
@@ -387,6 +465,44 @@ int Qwen3Decoder::enqueue_step_layers() {
         KX_LAYER(L.down->forward(act_, down_));
     }
     KX_LAYER(final_norm_op_->forward(x_, down_, h_));
+    KX_LAYER(lm_head_->forward(h_, logits_));
+#undef KX_LAYER
+    return kx_argmax_bf16(u16(logits_), c.vocab, io_.ptr<int32_t>() + 2, stream());
+}
+
+// The launches of enqueue_step_fused(), each as the forward() of a kuiper layer (the projections in their fused
+// form, set in attach_layer_weights()).  The first layer's row is normed by a stand-alone RmsNormLayer: the
+// embedding leaves no tile sums of squares for the fused form to start from.
+int Qwen3Decoder::enqueue_step_layers() {
+    const Qwen3Config& c = config_;
+#define KX_LAYER(call)                          \
+    do {                                        \
+        const base::Status layer_status = call; \
+        if (!layer_status) {                    \
+            LOG(ERROR) << layer_status.get_err_msg(); \
+            return KX_ERR_BAD_SHAPE;            \
+        }                                       \
+    } while (0)
+    KX_LAYER(embedding_op_->forward(token_view_, x_));
+    for (int32_t li = 0; li < c.layers; li++) {
+        LayerWeights& L = layers_[static_cast<size_t>(li)];
+        if (li == 0) {
+            KX_LAYER(layer_ops_[0].input_norm->forward(x_, h_));
+            L.qkv->set_input(0, h_);
+        }
+        KX_LAYER(L.qkv->forward());
+        if (merge_in_o_) {
+            KX_LAYER(attention_op_->forward_chunks(q_, pos_view_, L.k_cache, L.v_cache));
+        } else {
+            KX_LAYER(attention_op_->forward(q_, pos_view_, L.k_cache, L.v_cache, attn_));
+            L.o->set_input(0, attn_);
+        }
+        KX_LAYER(L.o->forward());
+        L.gate_up->set_output(0, gate_up_);
+        KX_LAYER(L.gate_up->forward());
+        KX_LAYER(L.down->forward());
+    }
+    KX_LAYER(final_norm_op_->forward(x_, h_));
     KX_LAYER(lm_head_->forward(h_, logits_));
 #undef KX_LAYER
     return kx_argmax_bf16(u16(logits_), c.vocab, io_.ptr<int32_t>() + 2, stream());

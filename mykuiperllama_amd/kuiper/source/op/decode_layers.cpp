@@ -256,6 +256,33 @@ base::Status MultiHeadAttention::forward() {
     return base::error::success();
 }
 
+base::Status MultiHeadAttention::forward_chunks(const tensor::Tensor& q, const tensor::Tensor& pos,
+                                                const tensor::Tensor& k_cache, const tensor::Tensor& v_cache) {
+    if (device_type_ != base::DeviceType::DeviceCUDA) {
+        return base::error::invalid_argument("mha: the unmerged chunks exist on the GPU only");
+    }
+    set_input(0, q);
+    set_input(1, pos);
+    set_input(2, k_cache);
+    set_input(3, v_cache);
+    // everything check() asks of the inputs; there is no output tensor in this form
+    if (n_q_ < 1 || n_kv_ < 1 || n_q_ % n_kv_ != 0 || n_q_ / n_kv_ > 16) {
+        return base::error::invalid_argument("The head counts of the mha layer are invalid.");
+    }
+    KX_RETURN_IF_BAD(expect(q, base::DataType::DataTypeBf16, static_cast<size_t>(n_q_) * kHeadDim, "query"));
+    KX_RETURN_IF_BAD(expect(pos, base::DataType::DataTypeInt32, 1, "pos"));
+    if (k_cache.is_empty() || k_cache.dims_size() != 3 || k_cache.get_dim(1) != n_kv_ || k_cache.get_dim(2) != kHeadDim ||
+        k_cache.get_dim(0) > 65536) {
+        return base::error::invalid_argument("The key cache must be [max_positions <= 65536, n_kv_heads, 128].");
+    }
+    KX_RETURN_IF_BAD(expect(k_cache, base::DataType::DataTypeBf16, k_cache.size(), "key cache"));
+    KX_RETURN_IF_BAD(expect(v_cache, base::DataType::DataTypeBf16, k_cache.size(), "value cache"));
+    const base::Status grown = grow_workspace(kx_attn_decode_workspace_bytes(n_q_, kHeadDim, k_cache.get_dim(0)));
+    if (!grown) return grown;
+    kernel::get_mha_kernel(device_type_)(q, k_cache, v_cache, pos, workspace_, tensor::Tensor(), n_q_, n_kv_, stream());
+    return base::error::success();
+}
+
 base::Status MultiHeadAttention::reserve(int32_t max_positions) {
     if (device_type_ != base::DeviceType::DeviceCUDA) return base::error::success();
     const size_t need = kx_attn_decode_workspace_bytes(n_q_, kHeadDim, max_positions);

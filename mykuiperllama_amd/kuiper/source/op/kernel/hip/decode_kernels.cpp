@@ -97,11 +97,19 @@ void mha_kernel_cu(const tensor::Tensor& q, const tensor::Tensor& k_cache, const
     expect_gpu(v_cache);
     expect_gpu(pos);
     expect_gpu(workspace);
-    expect_gpu(output);
     CHECK_EQ(q.size(), static_cast<size_t>(n_q_heads) * kHeadDim);
-    CHECK_EQ(output.size(), q.size());
     CHECK_EQ(k_cache.dims_size(), 3);
     const int32_t max_positions = k_cache.get_dim(0);
+    if (output.is_empty()) {  // the first stage alone: the chunks stay in the workspace for their consumer
+        const int rc = kx_attn_decode_partial_bf16(q.ptr<uint16_t>(), k_cache.ptr<uint16_t>(), v_cache.ptr<uint16_t>(),
+                                                   n_q_heads, n_kv_heads, kHeadDim, pos.ptr<int32_t>(), max_positions,
+                                                   const_cast<uint8_t*>(workspace.ptr<uint8_t>()),
+                                                   workspace.byte_size(), stream);
+        CHECK(rc == KX_OK) << "attention kernel launch failed: " << kx_error_string(rc);
+        return;
+    }
+    expect_gpu(output);
+    CHECK_EQ(output.size(), q.size());
     const int rc = kx_attn_decode_bf16(q.ptr<uint16_t>(), k_cache.ptr<uint16_t>(), v_cache.ptr<uint16_t>(),
                                        out_ptr(output), n_q_heads, n_kv_heads, kHeadDim, pos.ptr<int32_t>(),
                                        max_positions, const_cast<uint8_t*>(workspace.ptr<uint8_t>()),

@@ -6,6 +6,7 @@
 #include <map>
 #include <memory>
 
+#include "../kernel_interface.h"
 #include "kx_hip.h"
 
 namespace kernel {
@@ -156,6 +157,120 @@ void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qwe
                                     qzeros.ptr<int32_t>(), const_cast<uint16_t*>(output.ptr<uint16_t>()), M, K,
                                     N, group_size, ws, ws_bytes, stream);
     CHECK(rc == KX_OK) << "AWQ matmul kernel launch failed: " << kx_error_string(rc);
+}
+
+namespace {
+
+void expect_gpu_tensor(const tensor::Tensor& t, const char* what) {
+    CHECK_EQ(t.is_empty(), false) << what;
+    CHECK(t.device_type() == base::DeviceType::DeviceCUDA) << what;
+}
+
+uint16_t* u16_of(const tensor::Tensor& t) {
+    return const_cast<uint16_t*>(t.ptr<uint16_t>());
+}
+
+}  // namespace
+
+void matmul_chain_kernel_cu(const MatmulChain& chain, const tensor::Tensor& qweight, const tensor::Tensor& scales,
+                            const tensor::Tensor& qzeros, int32_t group_size, void* stream) {
+    expect_gpu_tensor(qweight, "qweight");
+    expect_gpu_tensor(scales, "scales");
+    expect_gpu_tensor(qzeros, "qzeros");
+    CHECK_EQ(qweight.dims_size(), 2);
+    CHECK_GT(group_size, 0);
+    const int32_t K = qweight.get_dim(0);
+    const int32_t N = qweight.get_dim(1) * 8;
+    CHECK_EQ(K % group_size, 0);
+    CHECK_EQ(scales.size(), static_cast<size_t>(K / group_size) * N);
+    CHECK_EQ(qzeros.size(), static_cast<size_t>(K / group_size) * (N / 8));
+
+    kx_chain_desc d{};
+    switch (chain.in) {
+        case MatmulChain::In::Row:
+            expect_gpu_tensor(chain.x, "activation row");
+            CHECK_EQ(chain.x.size(), static_cast<size_t>(K));
+            d.in_kind = KX_IN_ROW;
+            d.x = chain.x.ptr<uint16_t>();
+            break;
+        case MatmulChain::In::SwiGLU:
+            expect_gpu_tensor(chain.gate, "gate");
+            expect_gpu_tensor(chain.up, "up");
+            CHECK_EQ(chain.gate.size(), static_cast<size_t>(K));
+            CHECK_EQ(chain.up.size(), static_cast<size_t>(K));
+            d.in_kind = KX_IN_SWIGLU;
+            d.gate = chain.gate.ptr<uint16_t>();
+            d.up = chain.up.ptr<uint16_t>();
+            break;
+        case MatmulChain::In::AttentionChunks:
+            expect_gpu_tensor(chain.attention_chunks, "attention chunks");
+            d.in_kind = KX_IN_ATTN;
+            d.attn_workspace = chain.attention_chunks.ptr<uint8_t>();
+            d.attn_workspace_bytes = chain.attention_chunks.byte_size();
+            d.n_q_heads = chain.n_q_heads;
+            d.n_kv_heads = chain.n_kv_heads;
+            d.max_positions = chain.max_positions;
+            break;
+        case MatmulChain::In::NormFromTileSums:
+            expect_gpu_tensor(chain.norm_row, "row to normalise");
+            expect_gpu_tensor(chain.norm_tile_sumsq, "tile sums of squares");
+            expect_gpu_tensor(chain.norm_gain, "norm gain");
+            CHECK_EQ(chain.norm_row.size(), static_cast<size_t>(K));
+            CHECK_EQ(chain.norm_gain.size(), static_cast<size_t>(K));
+            CHECK_EQ(chain.norm_tile_sumsq.size(), static_cast<size_t>((K + 255) / 256) * 4);
+            d.in_kind = KX_IN_NORM;
+            d.norm_row = chain.norm_row.ptr<uint16_t>();
+            d.norm_sumsq = chain.norm_tile_sumsq.ptr<float>();
+            d.norm_parts = (K + 255) / 256;
+            d.norm_gain = chain.norm_gain.ptr<uint16_t>();
+            d.norm_eps = chain.norm_eps;
+            break;
+    }
+    switch (chain.out) {
+        case MatmulChain::Out::Row:
+            expect_gpu_tensor(chain.y, "output row");
+            CHECK_EQ(chain.y.size(), static_cast<size_t>(N));
+            d.out_kind = KX_OUT_ROW;
+            d.y = u16_of(chain.y);
+            break;
+        case MatmulChain::Out::Residual:
+            expect_gpu_tensor(chain.residual, "residual row");
+            expect_gpu_tensor(chain.tile_sumsq, "tile sums of squares");
+            CHECK_EQ(chain.residual.size(), static_cast<size_t>(N));
+            CHECK_EQ(chain.tile_sumsq.size(), static_cast<size_t>((N + 255) / 256) * 4);
+            d.out_kind = KX_OUT_RESIDUAL;
+            d.residual_in = chain.residual.ptr<uint16_t>();
+            d.residual_out = u16_of(chain.residual);
+            d.sumsq_out = const_cast<float*>(chain.tile_sumsq.ptr<float>());
+            break;
+        case MatmulChain::Out::QkvRope:
+            expect_gpu_tensor(chain.q_gain, "q gain");
+            expect_gpu_tensor(chain.k_gain, "k gain");
+            expect_gpu_tensor(chain.q_out, "q output");
+            expect_gpu_tensor(chain.k_cache, "key cache");
+            expect_gpu_tensor(chain.v_cache, "value cache");
+            expect_gpu_tensor(chain.pos, "position");
+            CHECK_EQ(chain.k_cache.dims_size(), 3);
+            CHECK_EQ(chain.v_cache.size(), chain.k_cache.size());
+            d.out_kind = KX_OUT_QKV_ROPE;
+            d.q_gain = chain.q_gain.ptr<uint16_t>();
+            d.k_gain = chain.k_gain.ptr<uint16_t>();
+            d.q_out = u16_of(chain.q_out);
+            d.k_cache = u16_of(chain.k_cache);
+            d.v_cache = u16_of(chain.v_cache);
+            d.pos = chain.pos.ptr<int32_t>();
+            d.rope_n_q_heads = chain.rope_n_q_heads;
+            d.rope_n_kv_heads = chain.rope_n_kv_heads;
+            d.cache_positions = chain.k_cache.get_dim(0);
+            d.rope_theta = chain.rope_theta;
+            d.qk_eps = chain.qk_eps;
+            break;
+    }
+    const size_t ws_bytes = kx_gemv_workspace_bytes(1, K, N);
+    void* ws = workspace_for(stream, ws_bytes);
+    const int rc = kx_gemv_awq_chain_bf16(&d, qweight.ptr<int32_t>(), scales.ptr<uint16_t>(), qzeros.ptr<int32_t>(), K, N,
+                                          group_size, ws, ws_bytes, stream);
+    CHECK(rc == KX_OK) << "fused AWQ matmul launch failed: " << kx_error_string(rc);
 }
 
 }  // namespace kernel

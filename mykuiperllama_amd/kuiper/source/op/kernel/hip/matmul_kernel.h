@@ -16,6 +16,11 @@ void matmul_kernel_awq_cu(const tensor::Tensor& input, const tensor::Tensor& qwe
                           const tensor::Tensor& scales, const tensor::Tensor& qzeros,
                           const tensor::Tensor& output, int32_t group_size, void* stream);
 
+struct MatmulChain;
+// One fused launch of a decoder layer (kx_gemv_awq_chain_bf16), one activation row.
+void matmul_chain_kernel_cu(const MatmulChain& chain, const tensor::Tensor& qweight, const tensor::Tensor& scales,
+                            const tensor::Tensor& qzeros, int32_t group_size, void* stream);
+
 // Releases every cached workspace (for orderly shutdown in tests).
 void matmul_release_workspaces();
 // Releases the workspace of one stream; whoever destroys a stream calls this first, so that a later

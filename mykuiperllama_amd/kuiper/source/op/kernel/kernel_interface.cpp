@@ -41,6 +41,15 @@ MatmulKernelAwq get_matmul_kernel_awq(base::DeviceType device_type) {
     return nullptr;
 }
 
+MatmulChainKernel get_matmul_chain_kernel(base::DeviceType device_type) {
+    switch (device_type) {
+        case base::DeviceType::DeviceCUDA: return matmul_chain_kernel_cu;
+        default: break;  // the fused launches exist on the GPU only; a host layer runs its operators one by one
+    }
+    LOG(FATAL) << "Unknown device type for get a fused matmul kernel.";
+    return nullptr;
+}
+
 #define KX_SELECT(Type, getter, cpu_fn, gpu_fn, what)                         \
     Type getter(base::DeviceType device_type) {                               \
         switch (device_type) {                                                \

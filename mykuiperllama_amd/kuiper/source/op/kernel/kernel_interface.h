@@ -25,6 +25,30 @@ using MatmulKernelAwq = void (*)(const tensor::Tensor& input, const tensor::Tens
                                  const tensor::Tensor& output, int32_t group_size, void* stream);
 MatmulKernelAwq get_matmul_kernel_awq(base::DeviceType device_type);
 
+// The quantised matmul with its neighbours of a decoder layer inside the launch: where the activations come
+// from and where the result goes (one activation row).  Tensors that a kind does not use stay empty.
+struct MatmulChain {
+    enum class In { Row, SwiGLU, AttentionChunks, NormFromTileSums };
+    enum class Out { Row, Residual, QkvRope };
+    In in = In::Row;
+    Out out = Out::Row;
+    tensor::Tensor x;                                 // In::Row: bf16 [K]
+    tensor::Tensor gate, up;                          // In::SwiGLU: bf16 [K] each, x = bf16(silu(gate)) * up
+    tensor::Tensor attention_chunks;                  // In::AttentionChunks: what MultiHeadAttention::forward_chunks left
+    int32_t n_q_heads = 0, n_kv_heads = 0, max_positions = 0;
+    tensor::Tensor norm_row, norm_tile_sumsq, norm_gain;  // In::NormFromTileSums: x = gain * bf16(row * rsqrt(mean + eps)),
+    float norm_eps = 0.0f;                                 // the row's sums of squares given per quarter of 256 columns
+    tensor::Tensor y;                                 // Out::Row: bf16 [N]
+    tensor::Tensor residual, tile_sumsq;              // Out::Residual: residual <- bf16(residual + bf16(y)) in place,
+                                                      // fp32 [ceil(N / 256), 4] sums of squares of the new row
+    tensor::Tensor q_gain, k_gain, q_out, k_cache, v_cache, pos;  // Out::QkvRope: as RoPEKernel below
+    int32_t rope_n_q_heads = 0, rope_n_kv_heads = 0;
+    float rope_theta = 0.0f, qk_eps = 0.0f;
+};
+using MatmulChainKernel = void (*)(const MatmulChain& chain, const tensor::Tensor& qweight, const tensor::Tensor& scales,
+                                   const tensor::Tensor& qzeros, int32_t group_size, void* stream);
+MatmulChainKernel get_matmul_chain_kernel(base::DeviceType device_type);
+
 // Decode-step operators (the layer slots LayerRMSNorm, LayerSwiGLU, LayerEmbedding, LayerRope,
 // LayerMHA of kuiper/include/op/layer.h:8-20); bf16 tensors, head_dim 128.
 // y = gain * bf16(r * rsqrt(mean(r^2) + eps)) over the last dimension; with a non-empty `delta` the
@@ -53,7 +77,8 @@ using RoPEKernel = void (*)(const tensor::Tensor& qkv, const tensor::Tensor& q_g
 RoPEKernel get_rope_kernel(base::DeviceType device_type);
 
 // grouped-query attention of one query position against cache rows 0 .. pos[0]; `workspace` (GPU only)
-// holds the per-chunk results
+// holds the per-chunk results; with an empty `output` the GPU kernel stops there (the chunks are then merged
+// by the consumer, MatmulChain::In::AttentionChunks)
 using MhaKernel = void (*)(const tensor::Tensor& q, const tensor::Tensor& k_cache, const tensor::Tensor& v_cache,
                            const tensor::Tensor& pos, const tensor::Tensor& workspace, const tensor::Tensor& output,
                            int32_t n_q_heads, int32_t n_kv_heads, void* stream);

@@ -151,7 +151,61 @@ base::Status MatmulLayer::check() const {
     return status;
 }
 
+base::Status MatmulLayer::set_fusion(const kernel::MatmulChain& chain) {
+    if (!is_quant_layer_ || device_type_ != base::DeviceType::DeviceCUDA) {
+        return base::error::invalid_argument("Only a GPU AWQ matmul layer has fused launches.");
+    }
+    fusion_ = std::make_shared<kernel::MatmulChain>(chain);
+    return base::error::success();
+}
+
+void MatmulLayer::clear_fusion() { fusion_.reset(); }
+bool MatmulLayer::fused() const { return fusion_ != nullptr; }
+
+// The weights are checked as in check(); the ends that stay plain rows are input 0 / output 0 of the layer, the
+// other operands are checked by the kernel wrapper, like those of every GPU kernel of this API.
+base::Status MatmulLayer::forward_fused() {
+    const int32_t N = dim0_, K = dim1_, G = group_size_;
+    if (G < 32 || G % 32 != 0 || K % G != 0 || N % 8 != 0) {
+        return base::error::invalid_argument(
+            "AWQ needs a group size that is a multiple of 32 and divides K, and N a multiple of 8.");
+    }
+    base::Status status = check_tensor_with_dim(get_weight(0), device_type_, base::DataType::DataTypeInt32, K, N / 8);
+    if (status) status = check_tensor_with_dim(get_weight(1), device_type_, base::DataType::DataTypeInt32, K / G, N / 8);
+    if (status) status = check_tensor_with_dim(scales_, device_type_, base::DataType::DataTypeFp16, K / G, N);
+    if (!status) {
+        LOG(ERROR) << "The weight tensor error in the matmul layer.";
+        return status;
+    }
+    kernel::MatmulChain chain = *fusion_;
+    if (chain.in == kernel::MatmulChain::In::Row) {
+        chain.x = get_input(0);
+        status = check_tensor(chain.x, device_type_, base::DataType::DataTypeBf16);
+        if (status && batch_of(chain.x, K) != 1) status = base::error::invalid_argument("A fused launch takes one row [K].");
+        if (!status) {
+            LOG(ERROR) << "The input tensor error in the matmul layer.";
+            return status;
+        }
+    }
+    if (chain.out == kernel::MatmulChain::Out::Row) {
+        chain.y = get_output(0);
+        status = check_tensor(chain.y, device_type_, base::DataType::DataTypeBf16);
+        if (status && batch_of(chain.y, N) != 1) status = base::error::invalid_argument("A fused launch writes one row [N].");
+        if (!status) {
+            LOG(ERROR) << "The output tensor error in the matmul layer.";
+            return status;
+        }
+    }
+    CHECK_NE(cuda_config_, nullptr);
+    kernel::get_matmul_chain_kernel(device_type_)(chain, get_weight(0), scales_, get_weight(1), group_size_,
+                                                  cuda_config_->stream());
+    return base::error::success();
+}
+
 base::Status MatmulLayer::forward() {
+    if (fusion_) {
+        return forward_fused();
+    }
     base::Status status = check();
     if (!status) {
         return status;

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../oracle/kx_oracle.h"
+#include "../../mykuiperllama_amd/kuiper/source/op/kernel/kernel_interface.h"
 #include "mini_test.h"
 #include "model/qwen3_decoder.h"
 #include "model/safetensors.h"
@@ -203,13 +204,55 @@ TEST_GPU(test_qwen3_decoder, random_init_depends_on_the_seed_only) {
     ASSERT_TRUE(ms > 0.0);
 }
 
-TEST_GPU(test_qwen3_decoder, layer_by_layer_path_agrees_with_the_fused_path) {
-    // Same weights, same tokens: one forward() per operator against the fused entry points.  The fused
-    // path adds up the sum of squares of the RMSNorm tile by tile, so the logits agree to rounding.
+TEST_GPU(test_qwen3_decoder, fused_layers_return_the_bits_of_the_fused_entry_points) {
+    // The five launches of a decoder layer as forward() calls of kuiper layers (MatmulLayer::set_fusion,
+    // MultiHeadAttention::forward_chunks) against the same launches made through the C ABI directly: the same
+    // kernels on the same operands, except that the first layer's row is normed by a launch of its own, which
+    // returns the bits of the norm inside the launch.
     model::Qwen3Decoder fused(tiny_config(), 64), layers(tiny_config(), 64, model::DecodePath::Layers);
     fused.init_random(11);
     layers.init_random(11);
     ASSERT_TRUE(layers.path() == model::DecodePath::Layers);
+    ASSERT_EQ(layers.launches_per_step(), fused.launches_per_step() + 1);
+    const int32_t tokens[] = {9, 400, 77, 1000, 3, 3};
+    for (int i = 0; i < 6; i++) {
+        int32_t a = -1, b = -2;
+        ASSERT_TRUE(bool(fused.step(tokens[i], i, &a)));
+        ASSERT_TRUE(bool(layers.step(tokens[i], i, &b)));
+        ASSERT_EQ(a, b);
+        const std::vector<uint16_t> la = fused.logits(), lb = layers.logits();
+        ASSERT_EQ(std::memcmp(la.data(), lb.data(), la.size() * 2), 0);
+    }
+    // and from a captured graph
+    model::Qwen3Decoder replayed(tiny_config(), 64, model::DecodePath::Layers);
+    replayed.init_random(11);
+    ASSERT_TRUE(bool(replayed.capture()));
+    for (int i = 0; i < 6; i++) {
+        int32_t a = -1, b = -2;
+        ASSERT_TRUE(bool(fused.step(tokens[i], i, &a)));
+        ASSERT_TRUE(bool(replayed.step(tokens[i], i, &b)));
+        ASSERT_EQ(a, b);
+        const std::vector<uint16_t> la = fused.logits(), lb = replayed.logits();
+        ASSERT_EQ(std::memcmp(la.data(), lb.data(), la.size() * 2), 0);
+    }
+}
+
+TEST_GPU(test_qwen3_decoder, a_fused_form_is_refused_where_it_does_not_exist) {
+    op::MatmulLayer host(base::DeviceType::DeviceCPU, 256, 256, true, 128);
+    op::MatmulLayer dense(base::DeviceType::DeviceCUDA, 256, 256, false);
+    kernel::MatmulChain chain;
+    ASSERT_FALSE(bool(host.set_fusion(chain)));
+    ASSERT_FALSE(bool(dense.set_fusion(chain)));
+    ASSERT_FALSE(host.fused());
+}
+
+TEST_GPU(test_qwen3_decoder, operator_by_operator_path_agrees_with_the_fused_path) {
+    // Same weights, same tokens: one forward() per operator against the fused entry points.  The fused
+    // path adds up the sum of squares of the RMSNorm tile by tile, so the logits agree to rounding.
+    model::Qwen3Decoder fused(tiny_config(), 64), layers(tiny_config(), 64, model::DecodePath::Operators);
+    fused.init_random(11);
+    layers.init_random(11);
+    ASSERT_TRUE(layers.path() == model::DecodePath::Operators);
     ASSERT_EQ(layers.launches_per_step(), 1 + 2 * 10 + 3);
     const int32_t tokens[] = {9, 400, 77, 1000, 3, 3};
     for (int i = 0; i < 6; i++) {
@@ -228,9 +271,9 @@ TEST_GPU(test_qwen3_decoder, layer_by_layer_path_agrees_with_the_fused_path) {
     }
 }
 
-TEST_GPU(test_qwen3_decoder, layer_by_layer_path_can_be_captured) {
-    model::Qwen3Decoder eager(tiny_config(), 40, model::DecodePath::Layers);
-    model::Qwen3Decoder replayed(tiny_config(), 40, model::DecodePath::Layers);
+TEST_GPU(test_qwen3_decoder, operator_by_operator_path_can_be_captured) {
+    model::Qwen3Decoder eager(tiny_config(), 40, model::DecodePath::Operators);
+    model::Qwen3Decoder replayed(tiny_config(), 40, model::DecodePath::Operators);
     eager.init_random(5);
     replayed.init_random(5);
     ASSERT_TRUE(bool(replayed.capture()));  // nothing may allocate while the stream is captured

@@ -80,8 +80,10 @@ def test_gemv_m1_matches_oracle(capi, torch, oracle, K, N):
     check_against_oracle(oracle, p, y)
 
 
-@pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 16])
-@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 1024), (12288, 4096), (4096, 12288), (4096, 24576)])
+@pytest.mark.parametrize("M,K,N", [(M, K, N) for M in (2, 3, 4, 5, 8, 16)
+                                   for K, N in [(4096, 4096), (4096, 1024), (12288, 4096), (4096, 12288), (4096, 24576)]] +
+                         # the 32B-shaped MLP: K = 25 600 takes the four-step MFMA plan from five rows on
+                         [(M, K, N) for M in (2, 8, 16) for K, N in [(5120, 51200), (25600, 5120)]])
 def test_gemv_small_batch_matches_oracle(capi, torch, oracle, M, K, N):
     p = synth.make_awq_problem(f"gemv_m{M}_{K}x{N}", M, K, N)
     y, _ = run_awq(capi, torch, p)

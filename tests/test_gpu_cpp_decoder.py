@@ -67,7 +67,7 @@ def parse(stdout):
 @pytest.mark.gpu
 @pytest.mark.parametrize("max_positions", [48, 6000])
 def test_cpp_decoder_built_from_layers_matches_the_unfused_python_step(tmp_path, oracle, max_positions):
-    """--layers: one kuiper layer forward() per operator; DecodeModel.step(fused=False) enqueues the same
+    """--operators: one kuiper layer forward() per operator; DecodeModel.step(fused=False) enqueues the same
     ten launches per decoder layer through the C ABI."""
     import torch
     from mykuiperllama_amd import decode
@@ -83,7 +83,7 @@ def test_cpp_decoder_built_from_layers_matches_the_unfused_python_step(tmp_path,
         torch.cuda.synchronize()
         logits = model.logits.view(torch.int16).cpu().numpy().tobytes()
         expected.append((pos, token, int(model.next_token.item()), fnv1a64(logits)))
-    for mode in (["--layers"], ["--layers", "--graph"]):
+    for mode in (["--operators"], ["--operators", "--graph"]):
         done = run_tool(mode + ["--max-positions", max_positions, path] + TOKENS)
         assert done.returncode == 0, done.stderr
         launches = model.launches_per_step(with_lm_head=True, fused=False)
@@ -119,6 +119,13 @@ def test_cpp_decoder_matches_the_python_driver_bit_for_bit(tmp_path, oracle, max
                f"kv heads {cfg.n_kv} vocab {cfg.vocab} group 128" in done.stderr
         launches = model.launches_per_step(with_lm_head=True, fused=True)
         assert f"{launches} launches per step" in done.stderr
+        assert parse(done.stdout) == expected, (mode, done.stderr)
+    # --layers: the same launches, each the forward() of a kuiper layer (the projections in their fused form); the
+    # first layer's row is normed by a launch of its own, which changes no bit
+    for mode in (["--layers"], ["--layers", "--graph"]):
+        done = run_tool(mode + ["--max-positions", max_positions, path] + TOKENS)
+        assert done.returncode == 0, done.stderr
+        assert f"{launches + 1} launches per step" in done.stderr
         assert parse(done.stdout) == expected, (mode, done.stderr)
 
 

@@ -74,7 +74,7 @@ def test_dequant_exhaustive_over_q_z_and_every_fp16_scale(capi, torch, oracle):
         assert np.array_equal(got[~nan_ref], ref[~nan_ref]), f"z={z}"
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 7, 16])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 7, 8, 9, 12, 16])  # 8 | 9: one block of sixteen columns | four blocks per workgroup
 @pytest.mark.parametrize("K,N", [(4096, 4096), (1024, 3000), (5120, 1001)])
 def test_bf16_gemv_matches_oracle(capi, torch, oracle, M, K, N):
     p = synth.make_bf16_problem(f"bf16_{M}_{K}x{N}", M, K, N)
@@ -90,7 +90,7 @@ def test_bf16_gemv_matches_oracle(capi, torch, oracle, M, K, N):
     assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 5, 16])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 12, 16])
 @pytest.mark.parametrize("K,N", [(8, 1), (40, 15), (1000, 17), (4104, 1001), (72, 64)])
 def test_bf16_gemv_ragged_shapes(capi, torch, oracle, M, K, N):
     """K that is a multiple of eight but not of a sweep or of a 32-element MFMA step, N below and just past a
@@ -103,6 +103,30 @@ def test_bf16_gemv_ragged_shapes(capi, torch, oracle, M, K, N):
     ref_rounded = H.bf16_to_f64(oracle.f32_to_bf16(ref64.astype(np.float32)))
     got = H.bf16_to_f64(H.bf16_bits(y, torch))
     assert np.isfinite(got).all()
+    assert H.rel_l2(got, ref_rounded) <= 1e-3
+    assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
+
+
+@pytest.mark.parametrize("M", [1, 16])
+def test_bf16_gemv_at_the_size_of_the_qwen3_lm_head(capi, torch, oracle, M):
+    """K = 4096, N = 151 936 (37 984 workgroups at one row): a strided subset of 4 748 output rows plus the rows
+    of the first and the last workgroups against the oracle, everything else checked to be finite."""
+    K, N = 4096, 151936
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(424242 + M)
+    w = (torch.randn((N, K), device="cuda", generator=gen) * 0.02).bfloat16()
+    x = torch.randn((M, K), device="cuda", generator=gen).bfloat16()
+    y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_bf16(x, w, y)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    rows = np.unique(np.concatenate([np.arange(0, N, 32), np.arange(0, 64), np.arange(N - 64, N)]))
+    assert len(rows) >= 4096
+    idx = torch.from_numpy(rows).cuda()
+    w_sub = H.bf16_bits(w.index_select(0, idx), torch)
+    ref64 = oracle.gemv_bf16_f64(H.bf16_bits(x, torch), w_sub)
+    ref_rounded = H.bf16_to_f64(oracle.f32_to_bf16(ref64.astype(np.float32)))
+    got = H.bf16_to_f64(H.bf16_bits(y.index_select(1, idx), torch))
     assert H.rel_l2(got, ref_rounded) <= 1e-3
     assert np.abs(got - ref_rounded).max() <= 2 * H.bf16_ulp_of(np.abs(ref64).max())
 
