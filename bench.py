@@ -19,9 +19,9 @@ Prints one JSON line:  value = algorithmic bytes of a step / time of a step, in 
                 rotation, same replay) with the GEMV's distance to it
   validated     after the timed region the outputs the last timed step left behind are compared with the CPU
                 oracle (fp64 evaluation rounded to bf16) on the same weight set: relative L2 per shape
-  kernel_variants  the same shapes at M = 1 under each kernel the library holds: the two it chooses from (vector
-                ALU, one-shot MFMA) and the two measured alternatives it keeps selectable (K-loop "stream-K" kernel,
-                wide-load kernel through LDS), microseconds per launch
+  kernel_variants  five shapes at M = 1 under the two forced kernel policies (1 = vector-ALU kernel, 2 = one-shot
+                MFMA kernel, both with the K tiles meeting through partial sums in memory), microseconds per launch;
+                per_shape holds the product's own launch (vector kernel, K tiles meeting in 64-bit fixed point)
   small_batch   configs[2]: M in {1, 2, 4, 8, 16} on three shapes, microseconds per launch of the
                 vector-ALU kernel and of the MFMA kernel (cold weights, same event timing)
   decode        configs[3] and configs[4]: tokens/s of a full decode step (Qwen3-8B, Qwen3-32B-shaped); under the
@@ -46,7 +46,7 @@ METRIC = "INT4 AWQ GEMV achieved HBM GB/s (% of 8 TB/s); Qwen3-8B decode tok/s"
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --probe`, each counter scaled by what it
 # reads for a 256 MiB copy (profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md).  Counters cannot be
 # read from inside this process, so the figure is carried over from that profile and named as such.
-TRAFFIC_BYTES_PER_LAUNCH = 15337180
+TRAFFIC_BYTES_PER_LAUNCH = 15349775
 TRAFFIC_SOURCE = "profiles/awq_gemv_qwen3_8b_projections_hbm_counters.md"
 
 

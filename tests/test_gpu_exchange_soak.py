@@ -17,7 +17,7 @@ LAUNCHES = 2000
 CHUNK = 100  # launches between comparisons
 
 
-@pytest.mark.parametrize("policy", [0, 2], ids=["by_shape", "mfma"])
+@pytest.mark.parametrize("policy", [0, 1, 2], ids=["by_shape", "vector_ordered", "mfma"])
 def test_two_thousand_launches_on_one_workspace_repeat_their_first_results(policy):
     import torch
     from mykuiperllama_amd import capi
