@@ -73,8 +73,10 @@ int kx_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 /* ------------------------------------------------------------------------------------------
  * Fused INT4 AWQ dequantise + GEMV:   y[m,n] = sum_k x[m,k] * (q[k,n] - z[k/G,n]) * s[k/G,n]
  *   x bf16 [M,K] row-major, y bf16 [M,N] row-major, fp32 accumulation, 1 <= M <= KX_MAX_BATCH.
- *   Deterministic: the reduction order is fixed by (M,K,N,G), so repeated launches are bitwise
- *   identical.  qweight/qzeros 4-byte aligned, scales and x 16-byte aligned, y 8-byte aligned.
+ *   Reproducible: repeated launches are bitwise identical.  At M = 1 the partial sums of the K ranges of a
+ *   column meet in 64-bit fixed point (one atomic add each: the order of arrival cannot matter), at M >= 2 as
+ *   fp32 in an order fixed by (M,K,N,G).  qweight/qzeros 4-byte aligned, scales and x 16-byte aligned, y
+ *   8-byte aligned.
  * Replaces: the GPU branch of the quantised matmul kernel that the reference's MatmulLayer
  * would fetch through kernel::get_matmul_kernel_awq(DeviceCUDA) (pattern:
  * kuiper/source/op/kernel/kernel_interface.cpp:6-14, call site pattern kuiper/source/op/add.cpp:47).
@@ -108,14 +110,16 @@ int kx_gemv_awq_bf16_static(const uint16_t* x, const int32_t* qweight, const uin
 /* ------------------------------------------------------------------------------------------
  * The same GEMV with the activations produced on the way in, for the decode step (one launch
  * instead of two; M <= KX_MAX_BATCH).  Rounding points are those of the stand-alone kernels further
- * down, so each call returns what the two separate calls return.
+ * down; the K ranges of a column are added as fp32 in a fixed order here, so at M = 1 a call agrees with the two
+ * separate calls to the rounding of that sum (kx_gemv_awq_bf16 adds them in fixed point there), at M >= 2 bit
+ * for bit.
  *
  *   kx_gemv_awq_swiglu_bf16:  x[m,k] = bf16( bf16(silu(gate[m,k])) * up[m,k] ),  y = x W
  *       gate, up bf16, rows act_ld elements apart (act_ld >= K; halves of one [M, 2K] tensor or two
- *       tensors), 2-byte aligned.  Bitwise kx_swiglu_bf16 followed by kx_gemv_awq_bf16 on the same kernel:
- *       the vector kernel at M = 1, and at M >= 2 the matrix-core kernel, as kx_gemv_awq_bf16 chooses it,
- *       provided gate and up are 16-byte aligned and act_ld is a multiple of 8 (otherwise M >= 2 stays on
- *       the vector kernel, two rows per workgroup).
+ *       tensors), 2-byte aligned.  The vector kernel at M = 1; at M >= 2 the matrix-core kernel, as
+ *       kx_gemv_awq_bf16 chooses it (then bitwise kx_swiglu_bf16 followed by kx_gemv_awq_bf16), provided gate
+ *       and up are 16-byte aligned and act_ld is a multiple of 8 (otherwise M >= 2 stays on the vector kernel,
+ *       two rows per workgroup).
  *   kx_gemv_awq_addnorm_bf16 runs on the vector kernel for every M (built for M = 1).
  *   kx_gemv_awq_addnorm_bf16: r = bf16(residual + delta)   (delta may be null: r = residual)
  *                             x = gain * bf16(r * rsqrt(mean_k(r^2) + eps)),  y = x W
