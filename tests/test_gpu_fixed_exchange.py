@@ -59,6 +59,19 @@ def test_one_row_ragged_shapes_match_the_oracle(capi, torch, oracle, K, N, G):
     check_against_oracle(oracle, p, y)
 
 
+@pytest.mark.parametrize("K,N", [(512, 32768), (512, 32776), (8064, 264), (8192, 264)])
+def test_shapes_at_the_limits_of_the_slot_area_match_the_oracle(capi, torch, oracle, K, N):
+    """32768 columns fill the zeroed area with slots and masks, eight more take the ordered exchange; 8064 rows are
+    63 K tiles of 128 rows, the most a slot can count, 8192 rows take workgroups of 256 rows."""
+    p = synth.make_awq_problem(f"fixed_limit_{K}x{N}", 1, K, N)
+    y, (x, qw, sc, qz, ws) = run_awq(capi, torch, p)
+    check_against_oracle(oracle, p, y)
+    y2 = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
+    capi.gemv_awq_bf16(x, qw, sc, qz, y2, p["group"], ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(H.bf16_bits(y2, torch), y)
+
+
 @pytest.mark.parametrize("K,N", [(4096, 1024), (4096, 4096), (12288, 4096), (5120, 10240)])
 def test_one_hot_rows_the_sample_does_not_see_are_exact(capi, torch, oracle, K, N):
     """x = e_k with k outside the sample: the unit is the smallest one, the one non-zero partial sum of every
