@@ -69,7 +69,7 @@ def parse_args():
     ap.add_argument("--lib", default=None,
                     help="time another build of the HIP library (e.g. lib/libkx_hip_ablate1.so from "
                          "`python -m mykuiperllama_amd.build --ablate 1`); its numbers attribute time, its results "
-                         "are wrong by construction, so validation and the decode steps are skipped")
+                         "are wrong by construction, so validation and the small-batch table are skipped")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection workload: one 256 MiB device copy (known traffic, for scaling the "
                          "counters) followed by a few cold launches per projection shape; prints no metric")
@@ -494,7 +494,7 @@ def main():
         out["kernel_variants"] = kernel_variants
     if small_batch is not None:
         out["small_batch"] = small_batch
-    if not args.no_decode and not profiling_build:
+    if not args.no_decode:  # also with --lib: the builds that cut the first attention stage short are timed here
         del sets
         torch.cuda.empty_cache()
         d8 = decode_benchmark(torch, "qwen3-8b", 4096, args.decode_steps, 8, args.eager,

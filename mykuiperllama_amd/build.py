@@ -10,7 +10,10 @@
 `python -m mykuiperllama_amd.build --ablate N` additionally builds lib/libkx_hip_ablateN.so, the HIP
 library with parts of the GEMV kernels compiled out (-DKX_ABLATE=N: 1 = no split-K exchange, 2 = loads
 only, 3 = loads and arithmetic but neither the reduction across lanes and waves nor the exchange, on the
-vector kernel's plain launch; the other kernels as with 1); `bench.py --lib` times it.  Its results are wrong by construction: it exists to attribute time.
+vector kernel's plain launch; the other kernels as with 1; 4, 5, 6 = the first attention stage cut short: 4 = loads
+only, 5 = through the softmax statistics and the arrival of the V rows, 6 = everything but the stores of the
+weighted sums, the GEMV kernels whole); `bench.py --lib` times it.  Its results are wrong by construction: it exists
+to attribute time.
 
 Everything lands under mykuiperllama_amd/lib/, in-tree, so that a snapshot of the repository
 carries the binaries to a machine that only runs them.

@@ -591,7 +591,7 @@ __global__ __launch_bounds__(WAVES * kWave) void awq_gemv_kernel(
     }
 
     __shared__ uint32_t s_prev;
-#if defined(KX_ABLATE) && KX_ABLATE >= 1
+#if defined(KX_ABLATE) && KX_ABLATE >= 1 && KX_ABLATE <= 3
     if (ktiles > 1) {  // profiling build: no exchange - every workgroup leaves its partial sums and is done
         const int col = ct * kTileCols + tid;
         if (tid < kTileCols && col < N) partials[static_cast<size_t>(kt) * M * N + col] = psum[0];

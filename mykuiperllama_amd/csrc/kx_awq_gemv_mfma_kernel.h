@@ -372,7 +372,7 @@ __global__ __launch_bounds__(WAVES * kWave, 2) void awq_gemv_mfma_kernel(
         }
     }
 
-#if defined(KX_ABLATE) && KX_ABLATE >= 1
+#if defined(KX_ABLATE) && KX_ABLATE >= 1 && KX_ABLATE <= 3
     if (ktiles > 1) {  // profiling build: no exchange - every workgroup leaves its partial sums and is done
         if (tid < kTileCols && own_col < N) partials[static_cast<size_t>(kt) * M * N + own_col] = psum[0];
         return;

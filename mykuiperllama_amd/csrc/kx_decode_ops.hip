@@ -225,6 +225,21 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // for *pos and the round trip for the rows one after the other.  Such a chunk runs through with
     // everything masked and reports max = -inf, sum = 0.
 
+#if defined(KX_ABLATE) && KX_ABLATE == 4
+    {  // profiling build: loads only - fold what arrived into one word and leave
+        uint32_t f = static_cast<uint32_t>(ctx);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) f ^= qraw[ks].x ^ qraw[ks].w;
+#pragma unroll
+        for (int t = 0; t < TPW; t++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) f ^= kraw[t][ks].x ^ kraw[t][ks].y ^ kraw[t][ks].z ^ kraw[t][ks].w;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) f ^= vraw[it].x ^ vraw[it].y ^ vraw[it].z ^ vraw[it].w;
+        if (f == 0x9E3779B9u) out_base[tid] = 1.0f;
+        return;
+    }
+#endif
     // pass 1: scores, in units of log 2 (the exponentials below and in the merge are the hardware's exp2)
     const float scale2 = scale * 1.44269504088896341f;
     const bool q_live = mc < G;
@@ -292,6 +307,15 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // tiles, the even dims and the odd ones, so that one dword read per position feeds both.  The weights are
     // fp32 and the operands bf16: a weight enters as its bf16 rounding plus the bf16 rounding of what that left
     // over, two MFMAs per step (error 2^-17 relative instead of 2^-9).
+#if defined(KX_ABLATE) && KX_ABLATE == 5
+    {  // profiling build: scores and statistics, then wait for the V rows and leave
+        uint32_t f = 0;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) f ^= vraw[it].x ^ vraw[it].y ^ vraw[it].z ^ vraw[it].w;
+        if (f == 0x9E3779B9u) out_base[tid] = s_score[0][tid % CHUNK];
+        return;
+    }
+#endif
     constexpr int KSTEPS = CHUNK / 32;
     static_assert(ITERS % 2 == 0 && KSTEPS % 2 == 0, "two halves of whole steps");
     f32x4v dacc[2];
@@ -347,6 +371,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_stage1(
     // One test on the kind of store and one on the lane's heads around all four stores: inside the loop they
     // had become two branches per store.  (A lane's four heads are all live or all past G when G is a multiple
     // of four; other groupings take the per-head test.)
+#if defined(KX_ABLATE) && KX_ABLATE == 6
+    // profiling build: everything but the stores of the weighted sums
+    if (dacc[0][0] + dacc[1][1] + dacc[0][2] + dacc[1][3] != 12345.678f) return;
+#endif
     const bool all_four = 4 * mb + 3 < G;
     const int dim0 = 32 * wave + 2 * mc;
     if (one_sequence && all_four) {
