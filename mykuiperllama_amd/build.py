@@ -7,7 +7,7 @@
   libkx_probe.so  measurement only: the streaming-read kernel bench.py uses as the floor (probe/*.hip)
   test_kuiper_asan  optional (--asan): the host API and its C++ tests with AddressSanitizer on the host code
 
-`python -m mykuiperllama_amd.build --ablate N` additionally builds lib/libkx_hip_ablateN.so, the HIP
+`python -m mykuiperllama_amd.build --ablate N` builds lib/libkx_hip_ablateN.so (only that), the HIP
 library with parts of the GEMV kernels compiled out (-DKX_ABLATE=N: 1 = no split-K exchange, 2 = loads
 only, 3 = loads and arithmetic but neither the reduction across lanes and waves nor the exchange, on the
 vector kernel's plain launch; the other kernels as with 1; 4, 5, 6 = the first attention stage cut short: 4 = loads
@@ -135,12 +135,15 @@ def build_all():
 if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser()
-    ap.add_argument("--ablate", type=int, default=0, help="also build lib/libkx_hip_ablateN.so (profiling only)")
+    ap.add_argument("--ablate", type=int, default=0,
+                    help="build lib/libkx_hip_ablateN.so (profiling only) and nothing else, so that several of these "
+                         "builds can run side by side")
     ap.add_argument("--asan", action="store_true", help="also build lib/test_kuiper_asan (host code under AddressSanitizer)")
     args = ap.parse_args()
-    build_all()
-    print("built:", KX_LIB, KUIPER_LIB if os.path.exists(KUIPER_LIB) else "", PROBE_LIB)
     if args.ablate:
         print("built:", build_kx(args.ablate))
+        raise SystemExit(0)
+    build_all()
+    print("built:", KX_LIB, KUIPER_LIB if os.path.exists(KUIPER_LIB) else "", PROBE_LIB)
     if args.asan:
         print("built:", build_kuiper_asan())
